@@ -1,0 +1,93 @@
+/*
+ * tilefusion_c.h - C ABI of the MI355X (gfx950) TileFusion hot path.
+ *
+ * Plain pointers and sizes only: every pointer is a device pointer owned by the caller,
+ * every entry point enqueues on the HIP stream handed in (a hipStream_t passed as void*,
+ * NULL = the null stream) and returns without synchronising.  Nothing is allocated on the
+ * device.  Return value: TF_OK or an error code; tf_last_error() gives the thread-local
+ * message of the last failing call.  No entry point ever calls exit().
+ *
+ * The reference exports its host launchers as `extern "C"` symbols that take
+ * `torch::Tensor&` (include/kernels/ops.hpp:36-58), which is not a C ABI; the entry points
+ * below are what a binding (src/torch_bind.cc:8-14) calls instead.
+ */
+#ifndef TILEFUSION_C_H_
+#define TILEFUSION_C_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TF_API __attribute__((visibility("default")))
+
+typedef enum {
+  TF_OK = 0,
+  TF_ERR_INVALID_ARG = 1, /* null pointer, non-positive size, tile that does not divide */
+  TF_ERR_UNSUPPORTED = 2, /* legal in the reference but not compiled into this library  */
+  TF_ERR_LDS = 3,         /* requested tile needs more than 160 KiB of LDS              */
+  TF_ERR_HIP = 4          /* a HIP runtime call failed; message holds hipGetErrorString */
+} tf_status_t;
+
+/* C[M,N] = A[M,K] * B[K,N], fp16 inputs, fp32 accumulate.
+ * A is row-major [M,K]; B is column-major K x N, i.e. a row-major [N,K] buffer; C is
+ * row-major [M,N], fp32 when c_is_f16 == 0 (the reference op) or fp16 otherwise (the
+ * reference benchmark variant).  tm/tn/tk/num_stages/pipeline_level are the reference's
+ * tile-size and pipelining arguments: validated (tm | M, tn | N, tk | K, stages 1..3,
+ * level 0..2) and otherwise treated as a hint - the library maps the call onto its own
+ * MFMA tilings.  K must be a multiple of 8.
+ * Replaces: tilefusion::kernels::gemm, src/kernels/gemm.cu:63-142
+ * (schema include/kernels/kernel_list.hpp:15-18). */
+TF_API int tf_gemm_f16(const void* A, const void* B, void* C, int c_is_f16, int64_t M,
+                       int64_t N, int64_t K, int tm, int tn, int tk, int num_stages,
+                       int pipeline_level, void* stream);
+
+/* D[M,P] = (A[M,K] * B[K,N]) * C[N,P]; fp16 in/out, fp32 accumulate, A*B rounded to fp16
+ * in registers and never written to memory.  A row-major [M,K]; B a row-major [N,K]
+ * buffer; C a row-major [P,N] buffer; D row-major [M,P].  `batch` independent problems are
+ * laid out back to back (A, D strided by M*K / M*P; B and C strided by N*K / P*N).
+ * K and N must be multiples of 32, P a multiple of 16.
+ * Replaces: tilefusion::kernels::fused_two_gemms, src/kernels/fused_two_gemms.cu:66-144
+ * (schema include/kernels/kernel_list.hpp:20-23). */
+TF_API int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, void* D,
+                                  int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P,
+                                  int tm, int tn, int tk, int tp, void* stream);
+
+/* O = softmax(scale * Q K^T (+ causal mask)) V for `batch` independent (batch x head)
+ * slices laid out back to back.  fp16 in/out, fp32 scores, fp32 running max / sum.
+ * Q [batch, Lq, D]; K [batch, Lkv, D]; V [batch, Lkv, Dv] when v_is_transposed == 0, or
+ * [batch, Dv, Lkv] when 1 (what the reference op receives, python/ops/flash_attention.py:74);
+ * O [batch, Lq, Dv].  Causal mask: key index > query index is masked
+ * (include/cell/mask.hpp:75-82).  D and Dv must be 128 or 64; Lkv a multiple of 16.
+ * Replaces: tilefusion::kernels::flash_attention, src/kernels/flash_attn.cu:58-152
+ * (schema include/kernels/kernel_list.hpp:25-30). */
+TF_API int tf_flash_attention_fwd_f16(const void* Q, const void* K, const void* V, void* O,
+                                      int64_t batch, int64_t Lq, int64_t Lkv, int64_t D,
+                                      int64_t Dv, int v_is_transposed, int tile_length_q,
+                                      int tile_length_kv, int tile_hidden_qk, int tile_hidden_v,
+                                      double softmax_scale, int causal, void* stream);
+
+/* Single-query (decoding) attention with the KV range split into `num_splits` chunks:
+ * kernel 1 writes per-split partial (o, max, sum) in fp32 into `workspace`, kernel 2 merges
+ * them with a log-sum-exp weighted sum into O.
+ * Q [batch_heads, D]; K, V [batch_heads, Lkv, D]; O [batch_heads, D]; D must be 128.
+ * All offsets are 64-bit (K alone has 2^31 elements at the benchmark size).
+ * No counterpart in the reference (it has no decoding kernel); built on the same online
+ * softmax algebra as include/kernels/flash_attention_device.cuh:257-301. */
+TF_API size_t tf_flash_decode_workspace_bytes(int64_t batch_heads, int64_t D, int num_splits);
+TF_API int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void* O,
+                               void* workspace, size_t workspace_bytes, int64_t batch_heads,
+                               int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
+                               void* stream);
+
+/* Message of the last failing call on this thread ("" if none). */
+TF_API const char* tf_last_error(void);
+/* Library version string, e.g. "tilefusion-mi355x 0.1.0 (gfx950)". */
+TF_API const char* tf_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TILEFUSION_C_H_ */

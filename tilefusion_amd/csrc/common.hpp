@@ -1,0 +1,69 @@
+// Shared host/device helpers for the gfx950 kernels: vector types, MFMA wrappers,
+// direct global->LDS loads, error reporting for the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "tilefusion_c.h"
+
+namespace tfk {
+
+using half_t = _Float16;
+using half2_t = _Float16 __attribute__((ext_vector_type(2)));
+using half4_t = _Float16 __attribute__((ext_vector_type(4)));
+using half8_t = _Float16 __attribute__((ext_vector_type(8)));
+using float4_t = float __attribute__((ext_vector_type(4)));
+using float16_t = float __attribute__((ext_vector_type(16)));
+using uint4_t = unsigned __attribute__((ext_vector_type(4)));
+using uint2_t = unsigned __attribute__((ext_vector_type(2)));
+
+constexpr int kWaveSize = 64;
+constexpr int kMaxLdsBytes = 160 * 1024;
+
+#define TFK_DEVICE __device__ __forceinline__
+
+// D(32x32) += A(32x16) * B(16x32).  Lane l supplies A[l%32][8*(l/32)+t] and
+// B[8*(l/32)+t][l%32], t = 0..7; accumulator register r of lane l is
+// D[8*(r/4) + 4*(l/32) + r%4][l%32].
+TFK_DEVICE float16_t mfma_32x32x16(half8_t a, half8_t b, float16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+// D(16x16) += A(16x32) * B(32x16).  Lane l supplies A[l%16][8*(l/16)+t] and
+// B[8*(l/16)+t][l%16]; accumulator register r of lane l is D[4*(l/16)+r][l%16].
+TFK_DEVICE float4_t mfma_16x16x32(half8_t a, half8_t b, float4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// 16 bytes per lane straight from global memory into LDS, bypassing VGPRs.  `lds_wave_base`
+// must be wave-uniform; lane l's 16 bytes land at lds_wave_base + 16*l.
+TFK_DEVICE void load_global_to_lds_16B(const void* gptr, void* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(
+      (const __attribute__((address_space(1))) void*)gptr,
+      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+
+TFK_DEVICE void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// ---- host side ---------------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what);
+
+#define TFK_HIP_TRY(expr)                                   \
+  do {                                                      \
+    hipError_t e__ = (expr);                                \
+    if (e__ != hipSuccess) return ::tfk::hip_fail(e__, #expr); \
+  } while (0)
+
+#define TFK_REQUIRE(cond, code, ...)  \
+  do {                                \
+    if (!(cond)) {                    \
+      ::tfk::set_error(__VA_ARGS__);  \
+      return (code);                  \
+    }                                 \
+  } while (0)
+
+}  // namespace tfk

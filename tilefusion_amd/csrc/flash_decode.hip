@@ -1,0 +1,200 @@
+// Split-KV flash-decoding for gfx950: single-query attention per (batch x head) slice with the
+// key/value range cut into `num_splits` chunks, followed by a log-sum-exp combine.
+//
+// No counterpart in the reference (it has no decoding kernel); the per-chunk algebra is the
+// online softmax of include/kernels/flash_attention_device.cuh:257-301 with one query row.
+// Both kernels are HBM-bound streaming kernels, MFMA is irrelevant (1 flop per byte):
+//   * split kernel: grid (num_splits, batch_heads), 4 wavefronts.  One key row of 128 fp16 is
+//     256 bytes = 16 lanes x 16 bytes, so a wavefront load instruction fetches 4 whole rows
+//     fully coalesced; every 16-lane group keeps its own running (max, sum, o[128]) over the
+//     rows it sees and only the final merge of the 16 groups of a workgroup goes through LDS.
+//     The dot product is v_dot2_f32_f16 + a 4-step DPP rotate-add inside the 16-lane row;
+//     a batch of 8 rows per group is loaded before any is consumed to keep >= 16 KiB per
+//     wavefront in flight;
+//   * combine kernel: grid batch_heads, 128 threads, merges the fp32 partials.
+// All offsets are 64-bit.
+#include "common.hpp"
+
+namespace tfk {
+namespace {
+
+constexpr int kD = 128;
+constexpr int kDecWaves = 4;
+constexpr int kDecThreads = kDecWaves * kWaveSize;
+constexpr int kRowsPerStep = kDecWaves * 4;  // rows one workgroup load step covers
+constexpr int kBatchRows = 8;                // rows per 16-lane group between max updates
+
+template <int CTRL>
+TFK_DEVICE float dpp_f32(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, false));
+}
+// Sum over the 16 lanes of a DPP row; every lane ends up with the total.
+TFK_DEVICE float row16_sum(float x) {
+  x += dpp_f32<0x128>(x);  // row_ror:8
+  x += dpp_f32<0x124>(x);  // row_ror:4
+  x += dpp_f32<0x122>(x);  // row_ror:2
+  x += dpp_f32<0x121>(x);  // row_ror:1
+  return x;
+}
+
+TFK_DEVICE float dot8(half8_t k, half8_t q) {
+  float acc = 0.f;
+  acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(k, k, 0, 1), __builtin_shufflevector(q, q, 0, 1), acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(k, k, 2, 3), __builtin_shufflevector(q, q, 2, 3), acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(k, k, 4, 5), __builtin_shufflevector(q, q, 4, 5), acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_shufflevector(k, k, 6, 7), __builtin_shufflevector(q, q, 6, 7), acc, false);
+  return acc;
+}
+
+// workspace: o_part [batch_heads][num_splits][kD] fp32, then ml_part [batch_heads][num_splits][2]
+__global__ __launch_bounds__(kDecThreads) void flash_decode_split_kernel(
+    const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
+    float* __restrict__ o_part, float* __restrict__ ml_part, int64_t Lkv, int num_splits,
+    int64_t chunk, float scale_log2) {
+  __shared__ float s_o[kDecThreads / 16][kD];
+  __shared__ float s_m[kDecThreads / 16], s_l[kDecThreads / 16];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, g4 = lane >> 4;
+  const int split = blockIdx.x;
+  const int64_t bh = blockIdx.y;
+  const int64_t row_begin = (int64_t)split * chunk;
+  const int64_t row_end = min(row_begin + chunk, Lkv);
+
+  const half_t* kbase = K + bh * Lkv * kD + 8 * l16;
+  const half_t* vbase = V + bh * Lkv * kD + 8 * l16;
+  const half8_t q8 = *reinterpret_cast<const half8_t*>(Q + bh * kD + 8 * l16);
+
+  float m_run = -INFINITY, l_run = 0.f;
+  float o[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = 0.f;
+
+  for (int64_t r0 = row_begin + wave * 4 + g4; r0 < row_end + 0; r0 += (int64_t)kBatchRows * kRowsPerStep) {
+    half8_t kv[kBatchRows], vv[kBatchRows];
+#pragma unroll
+    for (int u = 0; u < kBatchRows; ++u) {
+      const int64_t row = min(r0 + (int64_t)u * kRowsPerStep, Lkv - 1);
+      kv[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(kbase + row * kD));
+    }
+#pragma unroll
+    for (int u = 0; u < kBatchRows; ++u) {
+      const int64_t row = min(r0 + (int64_t)u * kRowsPerStep, Lkv - 1);
+      vv[u] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(vbase + row * kD));
+    }
+    float s[kBatchRows];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < kBatchRows; ++u) {
+      const float d = row16_sum(dot8(kv[u], q8)) * scale_log2;
+      s[u] = (r0 + (int64_t)u * kRowsPerStep < row_end) ? d : -INFINITY;
+      mx = fmaxf(mx, s[u]);
+    }
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_safe);
+    m_run = m_new;
+    l_run *= alpha;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] *= alpha;
+#pragma unroll
+    for (int u = 0; u < kBatchRows; ++u) {
+      const float p = __builtin_amdgcn_exp2f(s[u] - m_safe);
+      l_run += p;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) o[i] += p * (float)vv[u][i];
+    }
+  }
+
+  // merge the 16 lane groups of the workgroup
+  const int grp = tid >> 4;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s_o[grp][8 * l16 + i] = o[i];
+  if (l16 == 0) {
+    s_m[grp] = m_run;
+    s_l[grp] = l_run;
+  }
+  __syncthreads();
+  if (tid < kD) {
+    float big = -INFINITY;
+#pragma unroll
+    for (int g = 0; g < kDecThreads / 16; ++g) big = fmaxf(big, s_m[g]);
+    const float big_safe = (big == -INFINITY) ? 0.f : big;
+    float acc = 0.f, l = 0.f;
+#pragma unroll
+    for (int g = 0; g < kDecThreads / 16; ++g) {
+      const float w = __builtin_amdgcn_exp2f(s_m[g] - big_safe);
+      acc += w * s_o[g][tid];
+      l += w * s_l[g];
+    }
+    const int64_t idx = bh * num_splits + split;
+    o_part[idx * kD + tid] = acc;
+    if (tid == 0) {
+      ml_part[idx * 2] = big;
+      ml_part[idx * 2 + 1] = l;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kD) void flash_decode_combine_kernel(
+    const float* __restrict__ o_part, const float* __restrict__ ml_part, half_t* __restrict__ O,
+    int num_splits) {
+  const int64_t bh = blockIdx.x;
+  const int d = threadIdx.x;
+  const float* ml = ml_part + bh * num_splits * 2;
+  const float* op = o_part + bh * num_splits * kD + d;
+  float big = -INFINITY;
+  for (int s = 0; s < num_splits; ++s) big = fmaxf(big, ml[2 * s]);
+  float acc = 0.f, l = 0.f;
+#pragma unroll 8
+  for (int s = 0; s < num_splits; ++s) {
+    const float w = __builtin_amdgcn_exp2f(ml[2 * s] - big);
+    acc += w * op[(int64_t)s * kD];
+    l += w * ml[2 * s + 1];
+  }
+  O[bh * kD + d] = (half_t)(acc / l);
+}
+
+}  // namespace
+}  // namespace tfk
+
+extern "C" size_t tf_flash_decode_workspace_bytes(int64_t batch_heads, int64_t D, int num_splits) {
+  if (batch_heads <= 0 || D <= 0 || num_splits <= 0) return 0;
+  return (size_t)batch_heads * (size_t)num_splits * (size_t)(D + 2) * sizeof(float);
+}
+
+extern "C" int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void* O,
+                                   void* workspace, size_t workspace_bytes, int64_t batch_heads,
+                                   int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
+                                   void* stream) {
+  using namespace tfk;
+  TFK_REQUIRE(Q && K && V && O && workspace, TF_ERR_INVALID_ARG, "tf_flash_decode_f16: null pointer");
+  TFK_REQUIRE(batch_heads > 0 && Lkv > 0 && num_splits > 0, TF_ERR_INVALID_ARG,
+              "tf_flash_decode_f16: sizes must be positive");
+  TFK_REQUIRE(batch_heads < 65536 && num_splits <= 65536, TF_ERR_INVALID_ARG,
+              "tf_flash_decode_f16: batch_heads / num_splits too large");
+  TFK_REQUIRE(D == kD, TF_ERR_UNSUPPORTED, "tf_flash_decode_f16: head dim must be 128 (got %lld)",
+              (long long)D);
+  TFK_REQUIRE(softmax_scale == softmax_scale && softmax_scale - softmax_scale == 0.0,
+              TF_ERR_INVALID_ARG, "tf_flash_decode_f16: softmax_scale must be finite");
+  const size_t need = tf_flash_decode_workspace_bytes(batch_heads, D, num_splits);
+  TFK_REQUIRE(workspace_bytes >= need, TF_ERR_INVALID_ARG,
+              "tf_flash_decode_f16: workspace holds %zu bytes, %zu needed", workspace_bytes, need);
+  TFK_REQUIRE(((uintptr_t)workspace & 15) == 0, TF_ERR_INVALID_ARG,
+              "tf_flash_decode_f16: workspace must be 16-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* o_part = static_cast<float*>(workspace);
+  float* ml_part = o_part + (size_t)batch_heads * num_splits * kD;
+  const int64_t chunk = (Lkv + num_splits - 1) / num_splits;
+  const float scale_log2 = (float)(softmax_scale * 1.4426950408889634);
+  hipLaunchKernelGGL(flash_decode_split_kernel, dim3(num_splits, (unsigned)batch_heads),
+                     dim3(kDecThreads), 0, st, static_cast<const half_t*>(Q),
+                     static_cast<const half_t*>(K), static_cast<const half_t*>(V), o_part, ml_part,
+                     Lkv, num_splits, chunk, scale_log2);
+  TFK_HIP_TRY(hipGetLastError());
+  hipLaunchKernelGGL(flash_decode_combine_kernel, dim3((unsigned)batch_heads), dim3(kD), 0, st,
+                     o_part, ml_part, static_cast<half_t*>(O), num_splits);
+  TFK_HIP_TRY(hipGetLastError());
+  return TF_OK;
+}

@@ -1,0 +1,198 @@
+// Fused back-to-back GEMM for gfx950: D[M,P] = (A[M,K] * B[K,N]) * C[N,P], fp16 in/out, fp32
+// accumulate; the intermediate A*B lives only in registers (rounded to fp16 like the
+// reference does, include/kernels/fused_two_gemms_device.cuh:200).
+//
+// Counterpart of ke_fused_two_gemms (include/kernels/fused_two_gemms_device.cuh:114-214) and its
+// host launcher (src/kernels/fused_two_gemms.cu:66-144).  CDNA4 design:
+//   * one workgroup = 64 rows of A (4 wavefronts x 16 rows), v_mfma_f32_16x16x32_f16;
+//   * the first GEMM is computed transposed, S^T = B_buf * A^T, so that every lane ends up
+//     holding one row m of A*B: the 16x16 accumulator layout (lane -> column m, registers ->
+//     4 consecutive n) is, after fp16 conversion, exactly the A-operand fragment layout of
+//     the second MFMA up to a permutation of the reduction index, which the C-operand loads
+//     mirror.  No LDS round trip, no shuffles for the intermediate;
+//   * B and C chunks go global -> LDS directly (global_load_lds_dwordx4) into XOR-swizzled
+//     tiles shared by the 4 wavefronts; A fragments are private to a wavefront and are read
+//     straight from global memory into registers;
+//   * D is staged through LDS so that global stores are 16 bytes per lane along rows.
+#include "common.hpp"
+
+namespace tfk {
+namespace {
+
+constexpr int kRowsPerBlock = 64;
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * kWaveSize;
+
+// Physical 16-byte chunk for logical chunk c of `row` in a tile whose rows hold CH chunks.
+template <int CH>
+__host__ __device__ constexpr int swz(int row, int c) {
+  constexpr int kRowsPer256B = CH >= 16 ? 1 : 16 / CH;
+  return c ^ ((row / kRowsPer256B) % CH);
+}
+
+// Cooperative direct global->LDS copy of a [ROWS x COLS] fp16 tile (row stride `ld` elements
+// in global memory) into a swizzled LDS tile with COLS-element rows.
+template <int ROWS, int COLS>
+TFK_DEVICE void tile_to_lds(const half_t* __restrict__ g, size_t ld, char* lds, int wave, int lane) {
+  constexpr int CH = COLS / 8;
+  constexpr int kRowsPerInstr = 64 / CH;
+  constexpr int kInstr = ROWS * CH / 64;
+  static_assert(ROWS * CH % 64 == 0, "tile must be a whole number of 1 KiB wavefront loads");
+  for (int i = wave; i < kInstr; i += kWaves) {
+    const int row = i * kRowsPerInstr + lane / CH;
+    const int c = swz<CH>(row, lane % CH);
+    load_global_to_lds_16B(g + (size_t)row * ld + c * 8, lds + i * 1024);
+  }
+}
+
+template <int TN, int TP, int KC>
+__global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
+    const half_t* __restrict__ A, const half_t* __restrict__ B, const half_t* __restrict__ C,
+    half_t* __restrict__ D, int M, int N, int K, int P) {
+  constexpr int kBChunks = KC / 8;   // 16-byte chunks per sB row
+  constexpr int kCChunks = TN / 8;   // per sC row
+  constexpr int kKSteps = KC / 32;
+  constexpr int kNT = TN / 16;       // 16-wide n tiles of the first GEMM
+  constexpr int kPT = TP / 16;       // 16-wide p tiles of the second GEMM
+  __shared__ __attribute__((aligned(1024))) char sB[TN * KC * 2];
+  __shared__ __attribute__((aligned(1024))) char sC[TP * TN * 2 < 1024 ? 1024 : TP * TN * 2];
+  __shared__ __attribute__((aligned(16))) half_t sD[kRowsPerBlock * TP];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  const int m0 = blockIdx.x * kRowsPerBlock;
+  const int p0 = blockIdx.y * TP;
+  const size_t batch = blockIdx.z;
+  A += batch * (size_t)M * K;
+  B += batch * (size_t)N * K;
+  C += batch * (size_t)P * N;
+  D += batch * (size_t)M * P;
+
+  const int a_row = min(m0 + wave * 16 + lr, M - 1);  // clamped: rows past M are never stored
+  const half_t* a_ptr = A + (size_t)a_row * K + 8 * lg;
+
+  float4_t acc2[kPT];
+#pragma unroll
+  for (int pt = 0; pt < kPT; ++pt) acc2[pt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (int n0 = 0; n0 < N; n0 += TN) {
+    float4_t acc1[kNT];
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) acc1[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int k0 = 0; k0 < K; k0 += KC) {
+      __syncthreads();  // previous readers of sB / sC are done
+      tile_to_lds<TN, KC>(B + (size_t)n0 * K + k0, K, sB, wave, lane);
+      if (k0 == 0) tile_to_lds<TP, TN>(C + (size_t)p0 * N + n0, N, sC, wave, lane);
+      half8_t af[kKSteps];
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks)
+        af[ks] = *reinterpret_cast<const half8_t*>(a_ptr + k0 + ks * 32);
+      wait_vmem_all();
+      __syncthreads();
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks)
+#pragma unroll
+        for (int nt = 0; nt < kNT; ++nt) {
+          const int row = nt * 16 + lr;
+          const half8_t bf = *reinterpret_cast<const half8_t*>(
+              sB + row * KC * 2 + swz<kBChunks>(row, ks * 4 + lg) * 16);
+          // S^T tile: rows n (from B), columns m (from A)
+          acc1[nt] = mfma_16x16x32(bf, af[ks], acc1[nt]);
+        }
+    }
+
+    // Second GEMM.  Lane (m = lr, group lg) holds A*B[m][16*nt + 4*lg + r] in acc1[nt][r];
+    // reduction step s uses n = 32*s + {4*lg + 0..3, 16 + 4*lg + 0..3} as its 8 slots.
+#pragma unroll
+    for (int s = 0; s < TN / 32; ++s) {
+      half8_t pa;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pa[r] = (half_t)acc1[2 * s][r];
+        pa[4 + r] = (half_t)acc1[2 * s + 1][r];
+      }
+#pragma unroll
+      for (int pt = 0; pt < kPT; ++pt) {
+        const int row = pt * 16 + lr;
+        const char* base = sC + row * TN * 2 + (lg & 1) * 8;
+        const half4_t lo = *reinterpret_cast<const half4_t*>(base + swz<kCChunks>(row, 4 * s + (lg >> 1)) * 16);
+        const half4_t hi = *reinterpret_cast<const half4_t*>(base + swz<kCChunks>(row, 4 * s + 2 + (lg >> 1)) * 16);
+        half8_t cf;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          cf[r] = lo[r];
+          cf[4 + r] = hi[r];
+        }
+        acc2[pt] = mfma_16x16x32(pa, cf, acc2[pt]);
+      }
+    }
+  }
+
+  // Epilogue: acc2[pt][r] = D[m0 + 16*wave + 4*lg + r][p0 + 16*pt + lr]
+#pragma unroll
+  for (int pt = 0; pt < kPT; ++pt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      sD[(wave * 16 + 4 * lg + r) * TP + pt * 16 + lr] = (half_t)acc2[pt][r];
+  __syncthreads();
+  constexpr int kDChunks = TP / 8;
+  for (int f = tid; f < kRowsPerBlock * kDChunks; f += kThreads) {
+    const int row = f / kDChunks, c = f % kDChunks;
+    if (m0 + row < M)
+      *reinterpret_cast<uint4_t*>(D + (size_t)(m0 + row) * P + p0 + c * 8) =
+          *reinterpret_cast<const uint4_t*>(sD + row * TP + c * 8);
+  }
+}
+
+template <int TN, int TP, int KC>
+int launch(const void* A, const void* B, const void* C, void* D, int batch, int M, int N, int K,
+           int P, hipStream_t st) {
+  dim3 grid((M + kRowsPerBlock - 1) / kRowsPerBlock, P / TP, batch);
+  hipLaunchKernelGGL((fused_two_gemms_kernel<TN, TP, KC>), grid, dim3(kThreads), 0, st,
+                     static_cast<const half_t*>(A), static_cast<const half_t*>(B),
+                     static_cast<const half_t*>(C), static_cast<half_t*>(D), M, N, K, P);
+  TFK_HIP_TRY(hipGetLastError());
+  return TF_OK;
+}
+
+template <int TN, int TP>
+int pick_kc(const void* A, const void* B, const void* C, void* D, int batch, int M, int N, int K,
+            int P, hipStream_t st) {
+  if (K % 128 == 0) return launch<TN, TP, 128>(A, B, C, D, batch, M, N, K, P, st);
+  return launch<TN, TP, 32>(A, B, C, D, batch, M, N, K, P, st);
+}
+
+template <int TN>
+int pick_tp(const void* A, const void* B, const void* C, void* D, int batch, int M, int N, int K,
+            int P, hipStream_t st) {
+  if (P % 128 == 0) return pick_kc<TN, 128>(A, B, C, D, batch, M, N, K, P, st);
+  if (P % 64 == 0) return pick_kc<TN, 64>(A, B, C, D, batch, M, N, K, P, st);
+  return pick_kc<TN, 16>(A, B, C, D, batch, M, N, K, P, st);
+}
+
+}  // namespace
+}  // namespace tfk
+
+extern "C" int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, void* D,
+                                      int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P,
+                                      int tm, int tn, int tk, int tp, void* stream) {
+  using namespace tfk;
+  TFK_REQUIRE(A && B && C && D, TF_ERR_INVALID_ARG, "tf_fused_two_gemms_f16: null pointer");
+  TFK_REQUIRE(batch > 0 && M > 0 && N > 0 && K > 0 && P > 0, TF_ERR_INVALID_ARG,
+              "tf_fused_two_gemms_f16: sizes must be positive");
+  TFK_REQUIRE(batch < 65536 && M < (1 << 30) && N < (1 << 24) && K < (1 << 24) && P < (1 << 24),
+              TF_ERR_INVALID_ARG, "tf_fused_two_gemms_f16: dimension too large");
+  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0 && tp > 0, TF_ERR_INVALID_ARG,
+              "tf_fused_two_gemms_f16: tile sizes must be positive");
+  TFK_REQUIRE(M % tm == 0 && N % tn == 0 && K % tk == 0 && P % tp == 0, TF_ERR_INVALID_ARG,
+              "tf_fused_two_gemms_f16: tile [%d,%d,%d,%d] does not divide problem [%lld,%lld,%lld,%lld]",
+              tm, tn, tk, tp, (long long)M, (long long)N, (long long)K, (long long)P);
+  TFK_REQUIRE(K % 32 == 0 && N % 32 == 0 && P % 16 == 0, TF_ERR_UNSUPPORTED,
+              "tf_fused_two_gemms_f16: needs K %% 32 == 0, N %% 32 == 0, P %% 16 == 0 (got K=%lld N=%lld P=%lld)",
+              (long long)K, (long long)N, (long long)P);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (N % 128 == 0) return pick_tp<128>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
+  return pick_tp<32>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
+}
