@@ -1,0 +1,335 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X TileFusion hot path.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+One "step" is one pass of a hot-path kernel over one batch of synthetic input that is
+already resident in HBM.  The default workload is the configuration the headline metric is
+quoted on - the 4096^3 fp16 GEMM (fp32 accumulate, fp16 out); the other benchmark
+configurations (fused back-to-back GEMM, flash-attention forward +/- causal, split-KV
+flash-decoding) are measured in the same run and reported under "workloads".  Prints ONE
+JSON line.
+
+Timing: W untimed warm-up steps, then exactly K steps between two HIP events recorded on the
+stream the kernels are launched on, bracketed by torch.cuda.synchronize().  Input sets rotate
+so that consecutive launches do not hit the 256 MB last-level cache with the same operands.
+The roofline entry is algorithmic flops (or bytes) per launch divided by the measured average
+launch duration.  The CPU baseline is the fp32 torch oracle timed on this host.
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP16_TFLOPS = 2516.6   # 256 CU x 2.4 GHz x 4096 flop/clk/CU (dense fp16 MFMA, "2.5 PFLOP/s")
+PEAK_HBM_GBS = 8000.0       # HBM3E, 8 TB/s
+
+
+def _time_steps(fn, steps, warmup):
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        fn(warmup + i)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    return e0.elapsed_time(e1) / steps, wall / steps
+
+
+def _cpu_time(fn, reps=3):
+    fn()
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+class Gemm4096:
+    name = "gemm_fp16_4096x4096x4096"
+    metric, unit, bound = "gemm_fp16_tflops", "TFLOP/s", "mfma"
+    M = N = K = 4096
+    flops = 2.0 * 4096 ** 3
+    bytes = 3 * 4096 * 4096 * 2
+
+    def setup(self, dev):
+        import torch
+        import oracle
+        self.lib = _capi().load()
+        a, b = oracle.make_c2_gemm_inputs()
+        self.host = (a, b)
+        g = torch.Generator(device=dev).manual_seed(2)
+        s = 1.0 / 64.0
+        self.sets = [(a.to(dev), b.to(dev), torch.empty(4096, 4096, device=dev, dtype=torch.float16))]
+        for _ in range(3):  # 4 sets x 96 MiB > 256 MB of last-level cache
+            self.sets.append(((torch.randn(4096, 4096, device=dev, generator=g) * s).half(),
+                              (torch.randn(4096, 4096, device=dev, generator=g) * s).half(),
+                              torch.empty(4096, 4096, device=dev, dtype=torch.float16)))
+
+    def step(self, i):
+        import torch
+        a, b, c = self.sets[i % len(self.sets)]
+        st = torch.cuda.current_stream().cuda_stream
+        rc = self.lib.tf_gemm_f16(a.data_ptr(), b.data_ptr(), c.data_ptr(), 1, 4096, 4096, 4096, 64, 128, 128, 2, 1, st)
+        assert rc == 0, self.lib.tf_last_error()
+
+    def check(self):
+        import oracle
+        self.step(0)
+        return oracle.check_close(self.sets[0][2], oracle.gemm_ref(*self.host))
+
+    def cpu_baseline(self):
+        import torch
+        a32, b32 = self.host[0].float(), self.host[1].float()
+        t = _cpu_time(lambda: torch.matmul(a32, b32.T))
+        return {"value": self.flops / t / 1e12, "unit": "TFLOP/s", "sample": "full 4096^3 fp32 torch.matmul, best of 3"}
+
+    config = {"workload": "fp16 GEMM M=N=K=4096, A row-major, B col-major, fp32 accumulate, fp16 out",
+              "inputs": "N(0,1)/sqrt(K), seed 1002; 4 rotating operand sets"}
+
+
+class Fused:
+    name = "fused_two_gemms_16384x128x128x128"
+    metric, unit, bound = "fused_two_gemms_gbs", "GB/s", "hbm"
+    M, N, K, P = 16384, 128, 128, 128
+    flops = 2.0 * 2 * 16384 * 128 * 128
+    bytes = (16384 * 128 * 2 + 2 * 128 * 128) * 2
+
+    def setup(self, dev):
+        import torch
+        import oracle
+        self.lib = _capi().load()
+        a, b, c = oracle.make_c3_fused_inputs()
+        self.host = (a, b, c)
+        self.sets = []
+        for i in range(40):  # 40 x 8.4 MB > 256 MB
+            self.sets.append((a.to(dev) if i == 0 else torch.roll(a.to(dev), i, 0), b.to(dev), c.to(dev),
+                              torch.empty(16384, 128, device=dev, dtype=torch.float16)))
+
+    def step(self, i):
+        import torch
+        a, b, c, d = self.sets[i % len(self.sets)]
+        st = torch.cuda.current_stream().cuda_stream
+        rc = self.lib.tf_fused_two_gemms_f16(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), 1, self.M, self.N,
+                                             self.K, self.P, 64, 128, 128, 128, st)
+        assert rc == 0, self.lib.tf_last_error()
+
+    def check(self):
+        import oracle
+        self.step(0)
+        return oracle.check_close(self.sets[0][3], oracle.fused_two_gemms_ref(*self.host))
+
+    def cpu_baseline(self):
+        a, b, c = (t.float() for t in self.host)
+        t = _cpu_time(lambda: (a @ b.T) @ c.T)
+        return {"value": self.bytes / t / 1e9, "unit": "GB/s", "sample": "full problem, two fp32 torch.matmul, best of 3"}
+
+    config = {"workload": "fused (A[16384x128] @ B[128x128]) @ C[128x128], fp16 in/out, fp32 accumulate",
+              "inputs": "N(0,1)/sqrt(128), seed 1003; 40 rotating A/D sets"}
+
+
+class Attention:
+    unit, bound = "TFLOP/s", "mfma"
+    B, H, S, D = 2, 32, 4096, 128
+
+    def __init__(self, causal):
+        self.causal = causal
+        self.name = "flash_attention_fwd_b2_h32_s4096_d128" + ("_causal" if causal else "")
+        self.metric = "flash_attention_fwd_tflops" + ("_causal" if causal else "")
+        self.flops = 4.0 * 64 * 4096 * 4096 * 128 * (0.5 if causal else 1.0)
+        self.bytes = 4 * 64 * 4096 * 128 * 2
+        self.config = {"workload": "flash-attention fwd fp16 B=2 H=32 S=4096 D=128 %s, scale 1/sqrt(128), fp32 softmax stats"
+                       % ("causal" if causal else "non-causal"),
+                       "inputs": "N(0,1), seed 1004; V in natural [S, D] layout; 2 rotating Q/K/V/O sets"}
+
+    def setup(self, dev):
+        import torch
+        import oracle
+        self.lib = _capi().load()
+        q, k, v = oracle.make_c4_attention_inputs()
+        self.host = (q, k, v)
+        mk = lambda t: t.reshape(64, 4096, 128).to(dev)
+        self.sets = [(mk(q), mk(k), mk(v), torch.empty(64, 4096, 128, device=dev, dtype=torch.float16))]
+        self.sets.append((mk(k), mk(v), mk(q), torch.empty(64, 4096, 128, device=dev, dtype=torch.float16)))
+
+    def step(self, i):
+        import torch
+        q, k, v, o = self.sets[i % len(self.sets)]
+        st = torch.cuda.current_stream().cuda_stream
+        rc = self.lib.tf_flash_attention_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), 64, 4096, 4096,
+                                                 128, 128, 0, 128, 64, 128, 128, 1.0 / math.sqrt(128), int(self.causal), st)
+        assert rc == 0, self.lib.tf_last_error()
+
+    _sample = [(0, 0), (1, 31)]
+
+    def check(self):
+        import oracle
+        self.step(0)
+        q, k, v = self.host
+        o = self.sets[0][3].cpu().reshape(2, 32, 4096, 128)
+        worst = (True, 0.0, 0.0)
+        for b, h in self._sample:
+            ok, r, m = oracle.check_close(o[b, h], oracle.attention_ref(q[b, h], k[b, h], v[b, h], causal=self.causal))
+            worst = (worst[0] and ok, max(worst[1], r), max(worst[2], m))
+        return worst
+
+    def cpu_baseline(self):
+        import oracle
+        q, k, v = self.host
+        n = len(self._sample)
+
+        def run():
+            for b, h in self._sample:
+                oracle.attention_ref(q[b, h], k[b, h], v[b, h], causal=self.causal)
+        t = _cpu_time(run, reps=2)
+        return {"value": self.flops * n / 64 / t / 1e12, "unit": "TFLOP/s",
+                "sample": "%d of 64 (batch, head) slices, fp32 softmax(QK^T)V per slice, best of 2" % n}
+
+
+class Decode:
+    name = "flash_decode_b16_h32_kv32768_d128_splits64"
+    metric, unit, bound = "flash_decode_hbm_gbs", "GB/s", "hbm"
+    BH, LKV, D, SPLITS = 512, 32768, 128, 64
+    bytes = 2 * 512 * 32768 * 128 * 2 + 2 * 512 * 128 * 2
+    flops = 4.0 * 512 * 32768 * 128
+
+    def setup(self, dev):
+        import torch
+        import oracle
+        self.lib = _capi().load()
+        g = torch.Generator(device=dev).manual_seed(oracle.SEEDS["c5"])
+        self.q = torch.randn(self.BH, self.D, device=dev, dtype=torch.float16, generator=g)
+        self.k = torch.randn(self.BH, self.LKV, self.D, device=dev, dtype=torch.float16, generator=g)
+        self.v = torch.randn(self.BH, self.LKV, self.D, device=dev, dtype=torch.float16, generator=g)
+        self.o = torch.empty(self.BH, self.D, device=dev, dtype=torch.float16)
+        self.ws_bytes = self.lib.tf_flash_decode_workspace_bytes(self.BH, self.D, self.SPLITS)
+        self.ws = torch.empty(self.ws_bytes, device=dev, dtype=torch.uint8)
+
+    def step(self, i):
+        import torch
+        st = torch.cuda.current_stream().cuda_stream
+        rc = self.lib.tf_flash_decode_f16(self.q.data_ptr(), self.k.data_ptr(), self.v.data_ptr(), self.o.data_ptr(),
+                                          self.ws.data_ptr(), self.ws_bytes, self.BH, self.LKV, self.D, self.SPLITS,
+                                          1.0 / math.sqrt(self.D), st)
+        assert rc == 0, self.lib.tf_last_error()
+
+    _sample = [0, 100, 255, 511]
+
+    def check(self):
+        import oracle
+        self.step(0)
+        worst = (True, 0.0, 0.0)
+        for i in self._sample:
+            ok, r, m = oracle.check_close(self.o[i], oracle.flash_decode_ref(self.q[i].cpu(), self.k[i].cpu(), self.v[i].cpu()))
+            worst = (worst[0] and ok, max(worst[1], r), max(worst[2], m))
+        return worst
+
+    def cpu_baseline(self):
+        import oracle
+        host = [(self.q[i].cpu(), self.k[i].cpu(), self.v[i].cpu()) for i in self._sample]
+
+        def run():
+            for q, k, v in host:
+                oracle.flash_decode_ref(q, k, v)
+        t = _cpu_time(run)
+        return {"value": self.bytes * len(host) / self.BH / t / 1e9, "unit": "GB/s",
+                "sample": "%d of 512 (batch, head) slices, fp32 softmax(qK^T)V per slice, best of 3" % len(host)}
+
+    config = {"workload": "flash-decoding fp16 B=16 H=32 q_len=1 KV=32768 D=128, 64 splits + LSE combine (2 kernels per step)",
+              "inputs": "N(0,1) drawn on the device, seed 1005; 8 GiB of K,V (exceeds the last-level cache)"}
+
+
+def _capi():
+    from tilefusion_amd import _capi as m
+    return m
+
+
+def run_workload(w, steps, warmup, with_cpu):
+    import torch
+    dev = "cuda:0"
+    w.setup(dev)
+    ok, rel, mabs = w.check()
+    ms, wall_ms = _time_steps(w.step, steps, warmup)
+    if w.bound == "mfma":
+        achieved, peak, runit = w.flops / ms / 1e9, PEAK_FP16_TFLOPS, "TFLOP/s"
+    else:
+        achieved, peak, runit = w.bytes / ms / 1e6, PEAK_HBM_GBS, "GB/s"
+    out = {
+        "metric": w.metric, "value": round(achieved, 2), "unit": w.unit, "ms_per_step": round(ms, 5),
+        "wall_ms_per_step": round(wall_ms, 5),
+        "roofline": {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": runit,
+                     "frac": round(achieved / peak, 4), "traffic": None},
+        "tflops": round(w.flops / ms / 1e9, 2), "algorithmic_gbs": round(w.bytes / ms / 1e6, 1),
+        "parity": {"ok": bool(ok), "rel_l2": float("%.3e" % rel), "max_abs": float("%.3e" % mabs),
+                   "tolerance": "rel_l2<=1e-3, max_abs<=2e-2 vs fp32 CPU oracle"},
+        "config": w.config,
+    }
+    if with_cpu:
+        cb = w.cpu_baseline()
+        cb["value"] = round(cb["value"], 4)
+        cb["cores"] = torch.get_num_threads()
+        cb["kind"] = "port"
+        out["cpu_baseline"] = cb
+    del w
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "gemm", "fused", "attention", "attention_causal", "decode"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is not supported "
+              "(see DESIGN.md for how each kernel would shard).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))))
+    table = {"gemm": Gemm4096(), "fused": Fused(), "attention": Attention(False),
+             "attention_causal": Attention(True), "decode": Decode()}
+    head_key = "gemm" if args.workload == "all" else args.workload
+    head = run_workload(table[head_key], args.steps, args.warmup, not args.no_cpu)
+    prop = torch.cuda.get_device_properties(0)
+    line = {
+        "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
+        "parity": head["parity"],
+        "device": {"name": prop.name, "cus": prop.multi_processor_count, "host_cores": os.cpu_count()},
+    }
+    if "cpu_baseline" in head:
+        line["cpu_baseline"] = head["cpu_baseline"]
+    if args.workload == "all":
+        others = {}
+        for key in ("fused", "attention", "attention_causal", "decode"):
+            steps = args.steps if key != "decode" else max(5, min(args.steps, 20))
+            others[key] = run_workload(table[key], steps, min(args.warmup, 5), not args.no_cpu)
+        line["workloads"] = others
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

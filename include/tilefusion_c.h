@@ -60,7 +60,8 @@ TF_API int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, v
  * Q [batch, Lq, D]; K [batch, Lkv, D]; V [batch, Lkv, Dv] when v_is_transposed == 0, or
  * [batch, Dv, Lkv] when 1 (what the reference op receives, python/ops/flash_attention.py:74);
  * O [batch, Lq, Dv].  Causal mask: key index > query index is masked
- * (include/cell/mask.hpp:75-82).  D and Dv must be 128 or 64; Lkv a multiple of 16.
+ * (include/cell/mask.hpp:75-82).  (D, Dv) must be (128, 128) or (64, 64); any Lq and Lkv
+ * (a transposed V needs Lkv % 8 == 0 to keep its rows 16-byte aligned).
  * Replaces: tilefusion::kernels::flash_attention, src/kernels/flash_attn.cu:58-152
  * (schema include/kernels/kernel_list.hpp:25-30). */
 TF_API int tf_flash_attention_fwd_f16(const void* Q, const void* K, const void* V, void* O,

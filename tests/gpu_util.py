@@ -1,0 +1,64 @@
+"""Helpers shared by the GPU parity tests: call the C ABI on torch device buffers."""
+
+import math
+
+import torch
+
+from tilefusion_amd import _capi
+
+DEV = "cuda:0"
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def c_gemm(a, b, out_dtype=torch.float32, tiles=None, stages=1, level=0):
+    lib = _capi.load()
+    m, k = a.shape
+    n = b.shape[0]
+    tm, tn, tk = tiles if tiles else (m, n, k)
+    c = torch.full((m, n), float("nan"), device=a.device, dtype=out_dtype)
+    _capi.check(lib.tf_gemm_f16(a.data_ptr(), b.data_ptr(), c.data_ptr(), int(out_dtype == torch.float16),
+                                m, n, k, tm, tn, tk, stages, level, stream()), "tf_gemm_f16")
+    return c
+
+
+def c_fused(a, b, c, tiles=None):
+    lib = _capi.load()
+    batch = 1 if a.dim() == 2 else a.shape[0]
+    m, k = a.shape[-2:]
+    n, p = b.shape[-2], c.shape[-2]
+    tm, tn, tk, tp = tiles if tiles else (m, n, k, p)
+    d = torch.full((*a.shape[:-1], p), float("nan"), device=a.device, dtype=torch.float16)
+    _capi.check(lib.tf_fused_two_gemms_f16(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), batch,
+                                           m, n, k, p, tm, tn, tk, tp, stream()), "tf_fused_two_gemms_f16")
+    return d
+
+
+def c_attention(q, k, v, causal=False, scale=None, v_transposed=False, tiles=None):
+    """q [B, Lq, D], k [B, Lkv, D], v [B, Lkv, Dv] (or [B, Dv, Lkv] if v_transposed)."""
+    lib = _capi.load()
+    b, lq, d = q.shape
+    lkv = k.shape[1]
+    dv = v.shape[1] if v_transposed else v.shape[2]
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    t = tiles if tiles else (lq, lkv, d, dv)
+    o = torch.full((b, lq, dv), float("nan"), device=q.device, dtype=torch.float16)
+    _capi.check(lib.tf_flash_attention_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, lq, lkv,
+                                               d, dv, int(v_transposed), t[0], t[1], t[2], t[3], scale, int(causal),
+                                               stream()), "tf_flash_attention_fwd_f16")
+    return o
+
+
+def c_decode(q, k, v, num_splits, scale=None):
+    """q [BH, D], k, v [BH, Lkv, D]."""
+    lib = _capi.load()
+    bh, lkv, d = k.shape
+    scale = 1.0 / math.sqrt(d) if scale is None else scale
+    nbytes = lib.tf_flash_decode_workspace_bytes(bh, d, num_splits)
+    ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
+    o = torch.full((bh, d), float("nan"), device=q.device, dtype=torch.float16)
+    _capi.check(lib.tf_flash_decode_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(), nbytes,
+                                        bh, lkv, d, num_splits, scale, stream()), "tf_flash_decode_f16")
+    return o

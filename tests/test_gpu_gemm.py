@@ -1,0 +1,89 @@
+"""GPU parity of the GEMM macro kernel through the C ABI against the fp32 CPU oracle.
+Tolerance (benchmark contract): rel-L2 <= 1e-3 and max-abs <= 2e-2, fp16 in / fp32 accumulate."""
+
+import pytest
+import torch
+
+import oracle
+from oracle import numerics as N
+from tests.gpu_util import DEV, c_gemm
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(c, ref, what):
+    ok, r, m = N.check_close(c, ref)
+    assert ok, f"{what}: rel_l2={r:.3e} max_abs={m:.3e}"
+
+
+def test_readme_single_tile_gemm_c1():
+    # README example: A 128x256 row-major, B 256x64 col-major, C 128x64 fp32
+    a, b = oracle.make_c1_gemm_inputs()
+    c = c_gemm(a.to(DEV), b.to(DEV), torch.float32, (128, 64, 32))
+    _check(c, N.gemm_ref(a, b), "C1")
+    assert N.max_abs(c, N.gemm_ref(a, b)) < 1e-4  # fp32 output: only summation order differs
+
+
+# tests/python/test_gemm.py:75-135: (128^3, 256^3, 512^3) x tile 64^3 x (stages, level)
+@pytest.mark.parametrize("size,stages,level", [(128, 1, 0), (256, 1, 0), (256, 2, 1), (512, 2, 1), (512, 3, 2)])
+def test_reference_op_cases(size, stages, level):
+    g = torch.Generator().manual_seed(size + level)
+    a = torch.randn(size, size, generator=g).half()
+    b = torch.randn(size, size, generator=g).half()
+    c = c_gemm(a.to(DEV), b.to(DEV), torch.float32, (64, 64, 64), stages, level)
+    _check(c, N.gemm_ref(a, b), f"gemm {size}^3")
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_large_gemm_c2(out_dtype):
+    a, b = oracle.make_c2_gemm_inputs()
+    c = c_gemm(a.to(DEV), b.to(DEV), out_dtype, (64, 128, 128), 2, 1)
+    _check(c, N.gemm_ref(a, b), "C2 4096^3")
+
+
+# shapes of tests/cpp/cell/test_gemm.cu:316-375 (M,N in 16..128, K in 32..256) plus ragged
+# ones that exercise the bounds-checked path, non-square and mid-size direct-LDS tiles
+@pytest.mark.parametrize("m,n,k", [(16, 16, 32), (32, 32, 64), (64, 64, 128), (128, 128, 256), (64, 128, 64),
+                                   (100, 72, 40), (1, 1, 8), (33, 257, 136), (384, 128, 192), (256, 512, 64),
+                                   (1024, 768, 320), (2048, 256, 64)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_shapes(m, n, k, out_dtype):
+    g = torch.Generator().manual_seed(m * 131 + n * 17 + k)
+    a = torch.rand(m, k, generator=g).half()
+    b = torch.rand(n, k, generator=g).half()
+    c = c_gemm(a.to(DEV), b.to(DEV), out_dtype)
+    assert not torch.isnan(c).any()
+    ref = N.gemm_ref(a, b)
+    # U[0,1) inputs give outputs of size ~k/4: compare relative to that scale
+    assert N.rel_l2(c, ref) <= 1e-3
+    assert N.max_abs(c, ref) <= 2e-2 * max(1.0, float(ref.abs().max()))
+
+
+def test_integer_inputs_are_exact():
+    # products and sums of small integers are exact in fp32: bit-exact against the oracle
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(-3, 4, (512, 256), generator=g).half()
+    b = torch.randint(-3, 4, (384, 256), generator=g).half()
+    for dt in (torch.float32, torch.float16):
+        c = c_gemm(a.to(DEV), b.to(DEV), dt)
+        assert torch.equal(c.float().cpu(), N.gemm_ref(a, b))
+
+
+def test_linearity_at_full_size():
+    # size-independent property: (A1 + A2) B = A1 B + A2 B for integer-valued operands
+    g = torch.Generator(device=DEV).manual_seed(5)
+    a1 = torch.randint(-2, 3, (4096, 4096), generator=g, device=DEV).half()
+    a2 = torch.randint(-2, 3, (4096, 4096), generator=g, device=DEV).half()
+    b = torch.randint(-2, 3, (4096, 4096), generator=g, device=DEV).half()
+    assert torch.equal(c_gemm(a1 + a2, b), c_gemm(a1, b) + c_gemm(a2, b))
+
+
+def test_identity_operand():
+    g = torch.Generator().manual_seed(9)
+    a = torch.randn(256, 256, generator=g).half()
+    eye = torch.eye(256).half()
+    assert torch.equal(c_gemm(a.to(DEV), eye.to(DEV), torch.float16).cpu(), a)
+    # B buffer is [N, K]: C = A @ B^T, so a non-symmetric B catches a transposed operand
+    b = torch.randn(256, 256, generator=g).half()
+    c = c_gemm(eye.to(DEV), b.to(DEV), torch.float16).cpu()
+    assert torch.equal(c, b.T)

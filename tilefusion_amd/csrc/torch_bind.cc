@@ -1,0 +1,229 @@
+// PyTorch operator bindings: registers torch.ops.tilefusion.{gemm, fused_two_gemms,
+// flash_attention, flash_attention_fwd, flash_decode} for the CUDA dispatch key (HIP tensors
+// are "cuda" tensors on PyTorch-ROCm) and forwards to the C ABI in tilefusion_c.h on the
+// caller's current stream.
+//
+// Mirrors the reference's registry + binding (include/kernel_registry.hpp:20-88,
+// include/kernels/kernel_list.hpp:11-30, src/torch_bind.cc:8-14): the first three schemas are
+// byte-identical so existing callers of torch.ops.tilefusion.* keep working.  Differences:
+// outputs may be fp16 for gemm, leading batch dimensions are accepted, dimensions are read
+// from the right axes for non-square problems, launches go to the current stream instead of
+// the null stream, and errors surface as c10::Error (RuntimeError) instead of exit().
+#include <ATen/ATen.h>
+#include <c10/hip/HIPStream.h>
+#include <torch/library.h>
+
+#include <functional>
+#include <vector>
+
+#include "tilefusion_c.h"
+
+namespace tilefusion {
+
+#define CHECK_CUDA(x) TORCH_CHECK((x).device().is_cuda(), #x " must be a CUDA tensor.")
+#define CHECK_CONTIGUOUS(x) TORCH_CHECK((x).is_contiguous(), #x " must be contiguous.")
+#define CHECK_INPUT(x) \
+  CHECK_CUDA(x);       \
+  CHECK_CONTIGUOUS(x)
+#define CHECK_HALF(x) TORCH_CHECK((x).scalar_type() == at::kHalf, #x " must be a float16 tensor.")
+
+namespace {
+
+void* current_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+void check_status(int status, const char* op) {
+  TORCH_CHECK(status == TF_OK, "tilefusion::", op, " failed (status ", status, "): ", tf_last_error());
+}
+
+int64_t leading_numel(const at::Tensor& t, int64_t keep) {
+  int64_t n = 1;
+  for (int64_t i = 0; i + keep < t.dim(); ++i) n *= t.size(i);
+  return n;
+}
+
+}  // namespace
+
+namespace kernels {
+
+// gemm(A [M,K], B [N,K] (= column-major K x N), C [M,N] fp32 or fp16)
+void gemm(const at::Tensor& A, const at::Tensor& B, at::Tensor& C, int64_t tm, int64_t tn,
+          int64_t tk, int64_t num_stages, int64_t pipeline_level) {
+  CHECK_INPUT(A);
+  CHECK_INPUT(B);
+  CHECK_INPUT(C);
+  CHECK_HALF(A);
+  CHECK_HALF(B);
+  TORCH_CHECK(C.scalar_type() == at::kFloat || C.scalar_type() == at::kHalf,
+              "C must be a float32 or float16 tensor.");
+  TORCH_CHECK(A.dim() == 2 && B.dim() == 2 && C.dim() == 2, "gemm expects 2-D tensors.");
+  const int64_t m = A.size(0), k = A.size(1), n = B.size(0);
+  TORCH_CHECK(B.size(1) == k, "B must be [N, K] (column-major K x N); got K = ", B.size(1),
+              " vs ", k);
+  TORCH_CHECK(C.size(0) == m && C.size(1) == n, "C must be [M, N].");
+  check_status(tf_gemm_f16(A.data_ptr(), B.data_ptr(), C.data_ptr(), C.scalar_type() == at::kHalf,
+                           m, n, k, (int)tm, (int)tn, (int)tk, (int)num_stages,
+                           (int)pipeline_level, current_stream()),
+               "gemm");
+}
+
+// fused_two_gemms(A [.., M,K], B [.., N,K], C [.., P,N], D [.., M,P])
+void fused_two_gemms(const at::Tensor& A, const at::Tensor& B, const at::Tensor& C, at::Tensor& D,
+                     int64_t tm, int64_t tn, int64_t tk, int64_t tp) {
+  CHECK_INPUT(A);
+  CHECK_INPUT(B);
+  CHECK_INPUT(C);
+  CHECK_INPUT(D);
+  CHECK_HALF(A);
+  CHECK_HALF(B);
+  CHECK_HALF(C);
+  CHECK_HALF(D);
+  TORCH_CHECK(A.dim() >= 2 && A.dim() == B.dim() && A.dim() == C.dim() && A.dim() == D.dim(),
+              "fused_two_gemms expects tensors of equal rank >= 2.");
+  const int64_t batch = leading_numel(A, 2);
+  const int64_t m = A.size(-2), k = A.size(-1), n = B.size(-2), p = C.size(-2);
+  TORCH_CHECK(B.size(-1) == k, "B must be [N, K].");
+  TORCH_CHECK(C.size(-1) == n, "C must be [P, N].");
+  TORCH_CHECK(D.size(-2) == m && D.size(-1) == p, "D must be [M, P].");
+  TORCH_CHECK(leading_numel(B, 2) == batch && leading_numel(C, 2) == batch &&
+                  leading_numel(D, 2) == batch,
+              "batch dimensions must match.");
+  check_status(tf_fused_two_gemms_f16(A.data_ptr(), B.data_ptr(), C.data_ptr(), D.data_ptr(), batch,
+                                      m, n, k, p, (int)tm, (int)tn, (int)tk, (int)tp,
+                                      current_stream()),
+               "fused_two_gemms");
+}
+
+namespace {
+void attention_impl(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V, at::Tensor& O,
+                    bool v_transposed, int64_t tq, int64_t tkv, int64_t thqk, int64_t thv,
+                    double softmax_scale, bool causal, const char* op) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(O);
+  CHECK_HALF(Q);
+  CHECK_HALF(K);
+  CHECK_HALF(V);
+  CHECK_HALF(O);
+  TORCH_CHECK(Q.dim() >= 2 && Q.dim() == K.dim() && Q.dim() == V.dim() && Q.dim() == O.dim(),
+              op, " expects tensors of equal rank >= 2.");
+  const int64_t batch = leading_numel(Q, 2);
+  const int64_t lq = Q.size(-2), d = Q.size(-1), lkv = K.size(-2);
+  const int64_t dv = v_transposed ? V.size(-2) : V.size(-1);
+  const int64_t v_len = v_transposed ? V.size(-1) : V.size(-2);
+  TORCH_CHECK(K.size(-1) == d, "K must be [Lkv, D].");
+  TORCH_CHECK(v_len == lkv, "V does not match the key length.");
+  TORCH_CHECK(O.size(-2) == lq && O.size(-1) == dv, "O must be [Lq, Dv].");
+  TORCH_CHECK(leading_numel(K, 2) == batch && leading_numel(V, 2) == batch &&
+                  leading_numel(O, 2) == batch,
+              "batch dimensions must match.");
+  check_status(tf_flash_attention_fwd_f16(Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(),
+                                          batch, lq, lkv, d, dv, v_transposed ? 1 : 0, (int)tq,
+                                          (int)tkv, (int)thqk, (int)thv, softmax_scale,
+                                          causal ? 1 : 0, current_stream()),
+               op);
+}
+}  // namespace
+
+// flash_attention(Q [.., Lq,D], K [.., Lkv,D], V [.., Dv,Lkv] (transposed, as the reference's
+// Python wrapper passes it), O [.., Lq,Dv])
+void flash_attention(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V, at::Tensor& O,
+                     int64_t tile_length_q, int64_t tile_length_kv, int64_t tile_hidden_qk,
+                     int64_t tile_hidden_v, double softmax_scale, bool causal) {
+  attention_impl(Q, K, V, O, true, tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v,
+                 softmax_scale, causal, "flash_attention");
+}
+
+// flash_attention_fwd: same computation with V in its natural [.., Lkv, Dv] layout.
+void flash_attention_fwd(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V,
+                         at::Tensor& O, double softmax_scale, bool causal) {
+  attention_impl(Q, K, V, O, false, 1, 1, 1, 1, softmax_scale, causal, "flash_attention_fwd");
+}
+
+// flash_decode(Q [.., D], K [.., Lkv, D], V [.., Lkv, D], O [.., D]); the fp32 split-KV
+// partials live in a torch-allocated workspace.
+void flash_decode(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V, at::Tensor& O,
+                  int64_t num_splits, double softmax_scale) {
+  CHECK_INPUT(Q);
+  CHECK_INPUT(K);
+  CHECK_INPUT(V);
+  CHECK_INPUT(O);
+  CHECK_HALF(Q);
+  CHECK_HALF(K);
+  CHECK_HALF(V);
+  CHECK_HALF(O);
+  TORCH_CHECK(K.dim() >= 2 && V.dim() == K.dim(), "flash_decode: K and V must be [.., Lkv, D].");
+  const int64_t d = K.size(-1), lkv = K.size(-2);
+  const int64_t bh = leading_numel(K, 2);
+  TORCH_CHECK(V.size(-1) == d && V.size(-2) == lkv && leading_numel(V, 2) == bh,
+              "flash_decode: V must have the shape of K.");
+  TORCH_CHECK(Q.numel() == bh * d && O.numel() == bh * d,
+              "flash_decode: Q and O must hold one row of D per (batch, head).");
+  TORCH_CHECK(num_splits > 0, "flash_decode: num_splits must be positive.");
+  const size_t bytes = tf_flash_decode_workspace_bytes(bh, d, (int)num_splits);
+  at::Tensor ws = at::empty({(int64_t)((bytes + 3) / 4)}, Q.options().dtype(at::kFloat));
+  check_status(tf_flash_decode_f16(Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(),
+                                   ws.data_ptr(), bytes, bh, lkv, d, (int)num_splits, softmax_scale,
+                                   current_stream()),
+               "flash_decode");
+}
+
+}  // namespace kernels
+
+// Self-registering op table: each REGISTER_OP adds (schema, installer) at load time, and the
+// two TORCH_LIBRARY blocks below walk the table, like the reference's KernelRegistry.
+class KernelRegistry {
+ public:
+  using Installer = std::function<void(torch::Library&)>;
+  static KernelRegistry& instance() {
+    static KernelRegistry r;
+    return r;
+  }
+  template <typename Fn>
+  bool add_kernel(const char* name, const char* schema, Fn fn) {
+    schemas_.push_back(schema);
+    installers_.push_back([name, fn](torch::Library& m) { m.impl(name, c10::DispatchKey::CUDA, fn); });
+    return true;
+  }
+  void register_with_torch(torch::Library& m) const {
+    for (const char* s : schemas_) m.def(s);
+  }
+  void register_implementations(torch::Library& m) const {
+    for (const auto& f : installers_) f(m);
+  }
+
+ private:
+  std::vector<const char*> schemas_;
+  std::vector<Installer> installers_;
+};
+
+#define REGISTER_OP(name, schema, func) \
+  static const bool name##_registered = KernelRegistry::instance().add_kernel(#name, schema, func)
+
+REGISTER_OP(gemm,
+            "gemm(Tensor A, Tensor B, Tensor(a!) C, int m, int n, int k, "
+            "int num_stages, int pipeline_level) -> ()",
+            &kernels::gemm);
+REGISTER_OP(fused_two_gemms,
+            "fused_two_gemms(Tensor A, Tensor B, Tensor C, Tensor(a!) D, "
+            "int tm, int tn, int tk, int tp) ->()",
+            &kernels::fused_two_gemms);
+REGISTER_OP(flash_attention,
+            "flash_attention(Tensor Q, Tensor K, Tensor V, Tensor(a!) O, "
+            "int tile_length_q, int tile_length_kv, "
+            "int tile_hidden_qk, int tile_hidden_v, "
+            "float softmax_scale, bool causal) -> ()",
+            &kernels::flash_attention);
+REGISTER_OP(flash_attention_fwd,
+            "flash_attention_fwd(Tensor Q, Tensor K, Tensor V, Tensor(a!) O, "
+            "float softmax_scale, bool causal) -> ()",
+            &kernels::flash_attention_fwd);
+REGISTER_OP(flash_decode,
+            "flash_decode(Tensor Q, Tensor K, Tensor V, Tensor(a!) O, "
+            "int num_splits, float softmax_scale) -> ()",
+            &kernels::flash_decode);
+
+TORCH_LIBRARY(tilefusion, m) { KernelRegistry::instance().register_with_torch(m); }
+TORCH_LIBRARY_IMPL(tilefusion, CUDA, m) { KernelRegistry::instance().register_implementations(m); }
+
+}  // namespace tilefusion
