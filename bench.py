@@ -32,8 +32,21 @@ PEAK_FP16_TFLOPS = 2516.6   # 256 CU x 2.4 GHz x 4096 flop/clk/CU (dense fp16 MF
 PEAK_HBM_GBS = 8000.0       # HBM3E, 8 TB/s
 
 
+PRE_WARM_MS = 150.0  # the GPU takes ~100 ms of sustained load to settle its clocks
+
+
 def _time_steps(fn, steps, warmup):
     import torch
+    # Untimed pre-warm so that the W warm-up steps start from settled clocks: short benchmarks
+    # otherwise time the power-management ramp (first ~100 ms are 10-20% slower).
+    t_end = time.perf_counter() + PRE_WARM_MS / 1e3
+    i = 0
+    while time.perf_counter() < t_end:
+        fn(i)
+        i += 1
+        if i % 16 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()

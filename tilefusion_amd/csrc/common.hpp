@@ -47,6 +47,27 @@ TFK_DEVICE void load_global_to_lds_16B(const void* gptr, void* lds_wave_base) {
 }
 
 TFK_DEVICE void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Wait until at most N of this wavefront's vector-memory loads are still outstanding
+// (loads complete in issue order, so the oldest ones are the ones that have landed).
+template <int N>
+TFK_DEVICE void wait_vmem() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// Workgroup barrier for a direct-to-LDS pipeline: waits for this wavefront's LDS reads and
+// for all but its N youngest vector-memory loads, then synchronises.  __syncthreads() would
+// drain every outstanding load (vmcnt(0)) and with it the tiles still in flight.
+template <int N>
+TFK_DEVICE void barrier_keep_vmem() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+// Workgroup barrier that only drains this wavefront's LDS traffic (reads and writes), leaving
+// global loads into registers in flight.
+TFK_DEVICE void barrier_lds_only() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 
 // ---- host side ---------------------------------------------------------------------------
 void set_error(const char* fmt, ...);

@@ -4,22 +4,25 @@
 // Counterpart of the reference's ke_gemm / ke_gemm_level1_pipeline / ke_gemm_level2_pipeline
 // (include/kernels/gemm_device.cuh:110-419) and its host launcher (src/kernels/gemm.cu:63-142),
 // re-designed for CDNA4:
-//   * 64-lane wavefronts, v_mfma_f32_32x32x16_f16 base tiles, accumulators in the unified
+//   * 64-lane wavefronts, v_mfma_f32_16x16x32_f16 base tiles, accumulators in the unified
 //     512-entry register file (one wavefront per SIMD, 128x128 per wavefront at the big tile);
 //   * both operands are K-contiguous, so an MFMA operand fragment is one 16-byte LDS read;
 //   * tiles go global -> LDS without passing through VGPRs (global_load_lds_dwordx4) into a
-//     double-buffered, XOR-swizzled LDS layout: a wavefront instruction always writes 1 KiB
+//     four-stage, XOR-swizzled LDS ring: a wavefront instruction always writes 1 KiB
 //     of consecutive LDS, so the swizzle is applied on the global (source) side;
 //   * workgroup -> tile map keeps the workgroups of one XCD (one L2) on a compact block of
 //     output tiles.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace tfk {
 namespace {
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_>
 struct GemmShape {
   static constexpr int BM = BM_, BN = BN_, BK = BK_;
+  static constexpr int kStages = STAGES_;  // LDS stages of the direct-load pipeline
   static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
   static constexpr int kWaves = WAVES_M * WAVES_N;
   static constexpr int kThreads = kWaves * kWaveSize;
@@ -69,8 +72,42 @@ TFK_DEVICE void store_out(OutT* p, float v) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast path: M % BM == 0, N % BN == 0, K % BK == 0.  Direct global->LDS, two LDS stages.
+// Fast path: M % BM == 0, N % BN == 0, K % 32 == 0.  Direct global->LDS ring, 16x16x32 MFMA.
 // ------------------------------------------------------------------------------------------
+// Tile shape of the fast path.  BK is fixed at 32: one v_mfma_f32_16x16x32_f16 consumes a whole
+// k-tile, a 16-row operand fragment is one contiguous 1 KiB of LDS, and a tile is 32 KiB at
+// 256 x 256 so that four of them are in the ring.  (Under realistic operand data the MFMA
+// rate on MI355X is set by power, and the 16x16x32 shape sustains ~17% more flop/s than
+// 32x32x16 for the same 128 x 128 wavefront tile.)
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_>
+struct DirectShape {
+  static constexpr int BM = BM_, BN = BN_, BK = BK_;
+  static constexpr int kKSteps = BK / 32;                     // MFMA k-steps per tile
+  static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+  static constexpr int kStages = STAGES_;
+  static constexpr int kWaves = WAVES_M * WAVES_N;
+  static constexpr int kThreads = kWaves * kWaveSize;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;  // tile of one wavefront
+  static constexpr int TM = WM / 16, TN = WN / 16;            // 16x16 MFMA tiles per wavefront
+  static constexpr int kChunks = BK / 8;                      // 16-byte chunks per tile row
+  static constexpr int kRowsPer256B = 16 / kChunks;           // rows sharing one pass over the banks
+  static constexpr int kRowsPerInstr = 64 / kChunks;          // rows one wavefront load covers
+  static constexpr int kABytes = BM * BK * 2;
+  static constexpr int kBBytes = BN * BK * 2;
+  static constexpr int kStageBytes = kABytes + kBBytes;
+  static constexpr int kAInstr = BM * kChunks / 64 / kWaves;  // 1 KiB loads per wavefront
+  static constexpr int kBInstr = BN * kChunks / 64 / kWaves;
+  static_assert(WM % 16 == 0 && WN % 16 == 0, "wavefront tile must be MFMA-sized");
+  static_assert((BM * kChunks) % (64 * kWaves) == 0 && (BN * kChunks) % (64 * kWaves) == 0,
+                "tile rows must split evenly over the wavefronts' 1 KiB loads");
+  // With 64-byte rows, rows r, r+4, r+8, r+12 share a bank group (with 128-byte rows: r, r+2,
+  // ...), so the chunk index is XORed with (row / kRowsPer256B) % kChunks: sixteen consecutive
+  // rows reading one logical chunk then cover all sixteen 16-byte bank groups.
+  __host__ __device__ static constexpr int swizzle(int row, int c) {
+    return c ^ ((row / kRowsPer256B) % kChunks);
+  }
+};
+
 template <typename S, typename OutT>
 __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
     const half_t* __restrict__ A, const half_t* __restrict__ B, OutT* __restrict__ C, int M,
@@ -85,10 +122,9 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
   const int wm = wave / S::WAVES_N, wn = wave % S::WAVES_N;
 
   // --- global -> LDS plan -----------------------------------------------------------------
-  // Wavefront instruction i of a tile covers rows [i*kRowsPerInstr, +kRowsPerInstr); lane l
-  // fills physical chunk l % kChunks of row i*kRowsPerInstr + l / kChunks.
-  constexpr int kAInstr = S::BM * S::kChunks / 64 / S::kWaves;  // per wavefront
-  constexpr int kBInstr = S::BN * S::kChunks / 64 / S::kWaves;
+  // Wavefront instruction i of a tile covers 16 rows; lane l fills physical chunk l % 4 of
+  // row 16*i + l / 4 and fetches the logical chunk that the swizzle maps there.
+  constexpr int kAInstr = S::kAInstr, kBInstr = S::kBInstr;
   const int ld_row = lane / S::kChunks;
   const int ld_pc = lane % S::kChunks;
   const char* a_tile = reinterpret_cast<const char*>(A + (size_t)m0 * K);
@@ -104,78 +140,157 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
     const int row = (wave + S::kWaves * t) * S::kRowsPerInstr + ld_row;
     b_goff[t] = (unsigned)row * (unsigned)K * 2u + (unsigned)S::swizzle(row, ld_pc) * 16u;
   }
-  auto issue_tile_loads = [&](int stage, int k0) {
-    char* sa = smem + stage * S::kStageBytes;
-    char* sb = sa + S::kABytes;
-    const char* ga = a_tile + (size_t)k0 * 2;
-    const char* gb = b_tile + (size_t)k0 * 2;
-#pragma unroll
-    for (int t = 0; t < kAInstr; ++t)
-      load_global_to_lds_16B(ga + a_goff[t], sa + (wave + S::kWaves * t) * 1024);
-#pragma unroll
-    for (int t = 0; t < kBInstr; ++t)
-      load_global_to_lds_16B(gb + b_goff[t], sb + (wave + S::kWaves * t) * 1024);
-  };
 
   // --- LDS -> register plan ---------------------------------------------------------------
-  // Fragment (i, kk) of A: lane l reads row wm*WM + 32*i + l%32, logical chunk 2*kk + l/32.
-  const int fr = lane & 31, fg = lane >> 5;
+  // Fragment i of A at k-step ks: lane l reads row wm*WM + 16*i + l%16, logical chunk
+  // 4*ks + l/16 (8 halves of k).
+  const int fr = lane & 15, fg = lane >> 4;
+  const int ra = wm * S::WM + fr, rb = wn * S::WN + fr;
   unsigned a_rd[S::kKSteps], b_rd[S::kKSteps];
 #pragma unroll
-  for (int kk = 0; kk < S::kKSteps; ++kk) {
-    const int ra = wm * S::WM + fr, rb = wn * S::WN + fr;
-    a_rd[kk] = ra * S::BK * 2 + S::swizzle(ra, 2 * kk + fg) * 16;
-    b_rd[kk] = rb * S::BK * 2 + S::swizzle(rb, 2 * kk + fg) * 16;
+  for (int ks = 0; ks < S::kKSteps; ++ks) {
+    a_rd[ks] = ra * S::BK * 2 + S::swizzle(ra, 4 * ks + fg) * 16;
+    b_rd[ks] = rb * S::BK * 2 + S::swizzle(rb, 4 * ks + fg) * 16;
   }
 
-  float16_t acc[S::TM][S::TN];
+  // acc[i][j][r] = C[m0 + wm*WM + 16*i + l%16][n0 + wn*WN + 16*j + 4*(l/16) + r]: the MFMA is
+  // issued with the B fragment as its row operand, so a lane owns 4 consecutive columns of
+  // one row of C and stores them with one 8- or 16-byte instruction.
+  float4_t acc[S::TM][S::TN];
 #pragma unroll
   for (int i = 0; i < S::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < S::TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    for (int j = 0; j < S::TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
+  // --- main loop --------------------------------------------------------------------------
+  // kStages LDS stages, two sets of fragment registers, and an explicit issue schedule.
+  // A loaded MI355X needs the better part of a microsecond from issuing a tile's global->LDS
+  // loads to having it in LDS - about the MFMA time of a k-tile - so tile kt+kStages-1 is
+  // requested while tile kt is multiplied.  A k-tile is TM "slots" of TN MFMAs.  Per slot the
+  // wavefront also issues its share of the 1 KiB global->LDS loads of the far tile and the
+  // LDS reads that fetch one A and one B fragment of the NEXT tile, so neither the LDS pipe
+  // nor the texture-address path ever sees a burst (a burst of loads blocks the wavefront's
+  // MFMA issue while the address FIFO drains).  One workgroup barrier per k-tile, at its
+  // start: by then tile kt+1 has landed (s_waitcnt vmcnt leaves only the younger tiles'
+  // loads outstanding) and every wavefront has read all of tile kt into registers, so stage
+  // kt is free for the next iteration's loads.
+  constexpr int kLoadsPerTile = kAInstr + kBInstr;
+  constexpr int NS = S::kStages;
+  constexpr int KS = S::kKSteps;
+  constexpr int kSlots = KS * S::TM;
+  constexpr int kBarrierSlot = (KS - 1) * S::TM;  // in front of the tile's last k-step
+  static_assert(S::TN <= S::TM && (NS >= 3 || (NS == 2 && KS == 2)),
+                "issue schedule: TN <= TM; >= 3 stages, or 2 stages of 2 k-steps");
+  // NS >= 3: every slot of iteration kt requests a piece of tile kt+NS-1 (stage of tile kt-1,
+  // free since the previous barrier).  NS == 2: the slots in front of the barrier request the
+  // second half of tile kt+1, the slots behind it the first half of tile kt+2 (into the stage
+  // this barrier frees).
+  auto first_load = [](int slot) constexpr {
+    if (NS >= 3) return slot * kLoadsPerTile / kSlots;
+    return slot < kBarrierSlot ? kLoadsPerTile / 2 + slot * (kLoadsPerTile / 2) / kBarrierSlot
+                               : (slot - kBarrierSlot) * (kLoadsPerTile / 2) / (kSlots - kBarrierSlot);
+  };
+  auto end_load = [&](int slot) constexpr {
+    if (NS >= 3) return (slot + 1) * kLoadsPerTile / kSlots;
+    return slot < kBarrierSlot ? kLoadsPerTile / 2 + (slot + 1) * (kLoadsPerTile / 2) / kBarrierSlot
+                               : (slot + 1 - kBarrierSlot) * (kLoadsPerTile / 2) / (kSlots - kBarrierSlot);
+  };
+  // loads that may still be in flight when tile kt+1 is needed
+  constexpr int kInFlightAtBarrier =
+      NS >= 3 ? (NS - 3) * kLoadsPerTile + kBarrierSlot * kLoadsPerTile / kSlots : 0;
   const int num_k_tiles = K / S::BK;
-  issue_tile_loads(0, 0);
-  wait_vmem_all();
-  __syncthreads();
+  half8_t af[2][S::TM], bf[2][S::TN];
 
-  for (int kt = 0; kt < num_k_tiles; ++kt) {
-    if (kt + 1 < num_k_tiles) issue_tile_loads((kt + 1) & 1, (kt + 1) * S::BK);
-    const char* sa = smem + (kt & 1) * S::kStageBytes;
-    const char* sb = sa + S::kABytes;
-#pragma unroll
-    for (int kk = 0; kk < S::kKSteps; ++kk) {
-      half8_t af[S::TM], bf[S::TN];
-#pragma unroll
-      for (int i = 0; i < S::TM; ++i)
-        af[i] = *reinterpret_cast<const half8_t*>(sa + a_rd[kk] + i * 32 * S::BK * 2);
-#pragma unroll
-      for (int j = 0; j < S::TN; ++j)
-        bf[j] = *reinterpret_cast<const half8_t*>(sb + b_rd[kk] + j * 32 * S::BK * 2);
-#pragma unroll
-      for (int i = 0; i < S::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma_32x32x16(af[i], bf[j], acc[i][j]);
+  auto issue_load = [&](int stage, int k0, int n) __attribute__((always_inline)) {
+    char* sa = smem + stage * S::kStageBytes;
+    if (n < kAInstr) {
+      load_global_to_lds_16B(a_tile + (size_t)k0 * 2 + a_goff[n], sa + (wave + S::kWaves * n) * 1024);
+    } else {
+      const int t = n - kAInstr;
+      load_global_to_lds_16B(b_tile + (size_t)k0 * 2 + b_goff[t],
+                             sa + S::kABytes + (wave + S::kWaves * t) * 1024);
     }
-    wait_vmem_all();
-    __syncthreads();
+  };
+  auto load_frags = [&](int stage, int ks, int buf, int i) __attribute__((always_inline)) {
+    const char* sa = smem + stage * S::kStageBytes;
+    const char* sb = sa + S::kABytes;
+    af[buf][i] = *reinterpret_cast<const half8_t*>(sa + a_rd[ks] + i * 16 * S::BK * 2);
+    if (i < S::TN) bf[buf][i] = *reinterpret_cast<const half8_t*>(sb + b_rd[ks] + i * 16 * S::BK * 2);
+  };
+  // Past the end the schedule keeps running on a clamped tile index: the extra loads land in
+  // a stage nobody reads again, which is cheaper than a branch per slot.
+  auto tile_k = [&](int t) __attribute__((always_inline)) { return min(t, num_k_tiles - 1) * S::BK; };
+
+  if constexpr (NS >= 3) {
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t)
+#pragma unroll
+      for (int n = 0; n < kLoadsPerTile; ++n) issue_load(t, tile_k(t), n);
+    barrier_keep_vmem<(NS - 2) * kLoadsPerTile>();
+  } else {
+#pragma unroll
+    for (int n = 0; n < kLoadsPerTile; ++n) issue_load(0, tile_k(0), n);
+#pragma unroll
+    for (int n = 0; n < kLoadsPerTile / 2; ++n) issue_load(1, tile_k(1), n);
+    barrier_keep_vmem<kLoadsPerTile / 2>();
   }
+#pragma unroll
+  for (int i = 0; i < S::TM; ++i) load_frags(0, 0, 0, i);
+
+  // (No branch may sit inside this loop: at every control-flow join the compiler drains the
+  // LDS-direct loads with vmcnt(0), which serialises the whole pipeline.)
+  auto iteration = [&](int kt, auto parity_c) __attribute__((always_inline)) {
+    // fragment set used by k-step ks of this tile (steps alternate sets across tiles)
+    constexpr int base = (KS % 2) ? decltype(parity_c)::value : 0;
+    const int stage = kt % NS;
+    const int stage_next = (kt + 1) % NS;
+#pragma unroll
+    for (int slot = 0; slot < kSlots; ++slot) {
+      const int ks = slot / S::TM, i = slot % S::TM;
+      const int cur = base ^ (ks & 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if (slot == kBarrierSlot) barrier_keep_vmem<kInFlightAtBarrier>();
+#pragma unroll
+      for (int n = first_load(slot); n < end_load(slot); ++n) {
+        if constexpr (NS >= 3) {
+          issue_load((kt + NS - 1) % NS, tile_k(kt + NS - 1), n);
+        } else {
+          if (slot < kBarrierSlot) issue_load(stage_next, tile_k(kt + 1), n);
+          else issue_load(stage, tile_k(kt + 2), n);
+        }
+      }
+      if (ks + 1 < KS) load_frags(stage, ks + 1, cur ^ 1, i);
+      else load_frags(stage_next, 0, cur ^ 1, i);
+#pragma unroll
+      for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma_16x16x32(bf[cur][j], af[cur][i], acc[i][j]);
+    }
+  };
+  int kt = 0;
+  for (; kt + 1 < num_k_tiles; kt += 2) {
+    iteration(kt, std::integral_constant<int, 0>{});
+    iteration(kt + 1, std::integral_constant<int, 1>{});
+  }
+  if (kt < num_k_tiles) iteration(kt, std::integral_constant<int, 0>{});
+  __builtin_amdgcn_sched_barrier(0);
+  wait_vmem_all();  // the clamped tail loads must not outlive the workgroup's LDS
 
   // --- epilogue ---------------------------------------------------------------------------
-  const int c_row0 = m0 + wm * S::WM + 4 * fg;
-  const int c_col0 = n0 + wn * S::WN + fr;
+  const int c_row0 = m0 + wm * S::WM + fr;
+  const int c_col0 = n0 + wn * S::WN + 4 * fg;
 #pragma unroll
   for (int i = 0; i < S::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < S::TN; ++j)
+    for (int j = 0; j < S::TN; ++j) {
+      OutT* dst = C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j;
+      if constexpr (sizeof(OutT) == 2) {
+        half4_t v;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = c_row0 + i * 32 + 8 * (r / 4) + (r % 4);
-        const int col = c_col0 + j * 32;
-        store_out(C + (size_t)row * N + col, acc[i][j][r]);
+        for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][r];
+        *reinterpret_cast<half4_t*>(dst) = v;
+      } else {
+        *reinterpret_cast<float4_t*>(dst) = acc[i][j];
       }
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -251,14 +366,17 @@ __global__ __launch_bounds__(S::kThreads) void gemm_guarded_kernel(
       }
 }
 
-using ShapeBig = GemmShape<256, 256, 64, 2, 2>;
-using ShapeMid = GemmShape<128, 128, 64, 2, 2>;
-using ShapeSmall = GemmShape<64, 64, 32, 2, 2>;
+#ifndef TFK_GEMM_BIG
+#define TFK_GEMM_BIG 256, 256, 32, 2, 2, 4
+#endif
+using ShapeBig = DirectShape<TFK_GEMM_BIG>;           // 4 x 32 KiB of LDS, 128x128 per wavefront
+using ShapeMid = DirectShape<128, 128, 32, 2, 2, 4>;      // 4 x 16 KiB, 64x64 per wavefront
+using ShapeSmall = GemmShape<64, 64, 32, 2, 2, 1>;    // bounds-checked path
 
 template <typename S, typename OutT>
 int launch_direct(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
   auto kern = gemm_direct_lds_kernel<S, OutT>;
-  constexpr int lds = 2 * S::kStageBytes;
+  constexpr int lds = S::kStages * S::kStageBytes;
   static_assert(lds <= kMaxLdsBytes, "tile does not fit in LDS");
   static thread_local int configured_dev = -1;
   int dev = 0;
@@ -288,9 +406,9 @@ int launch_guarded(const void* A, const void* B, void* C, int M, int N, int K, h
 
 template <typename OutT>
 int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
-  if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
+  if (M % 256 == 0 && N % 256 == 0 && K % ShapeBig::BK == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
     return launch_direct<ShapeBig, OutT>(A, B, C, M, N, K, st);
-  if (M % 128 == 0 && N % 128 == 0 && K % 64 == 0)
+  if (M % 128 == 0 && N % 128 == 0 && K % 32 == 0)
     return launch_direct<ShapeMid, OutT>(A, B, C, M, N, K, st);
   return launch_guarded<ShapeSmall, OutT>(A, B, C, M, N, K, st);
 }
