@@ -46,6 +46,21 @@ TFK_DEVICE void load_global_to_lds_16B(const void* gptr, void* lds_wave_base) {
       (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
+// Same transfer issued from inline assembly.  The compiler then does not model the write into
+// LDS at all, so it never drains these loads on its own (with the builtin it inserts
+// vmcnt(0) at every control-flow join after a load); ordering against LDS reads is entirely
+// the caller's job (wait_vmem / barrier_keep_vmem below).  `lds_addr` is the wave-uniform LDS
+// byte address of the 1 KiB destination.
+TFK_DEVICE void lds_dma_16B(const void* gptr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gptr), "s"(lds_addr)
+               : "memory");
+}
+TFK_DEVICE unsigned lds_address(const void* p) {
+  return (unsigned)(size_t)((__attribute__((address_space(3))) const char*)p);
+}
+
 TFK_DEVICE void wait_vmem_all() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 // Wait until at most N of this wavefront's vector-memory loads are still outstanding
 // (loads complete in issue order, so the oldest ones are the ones that have landed).

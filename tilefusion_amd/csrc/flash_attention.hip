@@ -4,26 +4,26 @@
 // Counterpart of ke_flash_attention (include/kernels/flash_attention_device.cuh:130-312, mask
 // include/cell/mask.hpp:75-82) and its host launcher (src/kernels/flash_attn.cu:58-152).
 // CDNA4 design (FA-2 style, un-normalised O with one divide at the end):
-//   * one workgroup = 128 queries (4 wavefronts x 32), key/value tiles of 64 rows,
-//     v_mfma_f32_32x32x16_f16 throughout;
+//   * one workgroup = 256 queries (8 wavefronts x 32; 4 x 32 for short query ranges),
+//     key/value tiles of 64 rows, v_mfma_f32_32x32x16_f16 throughout;
 //   * Q stays in registers for the whole workgroup (the reference reloads it per KV tile);
 //   * scores are computed transposed, S^T = K Q^T, so a lane owns ONE query row: its 32
 //     score values per tile are plain registers, the row max / sum is an in-lane reduction
 //     plus a single v_permlane32_swap with the partner lane, and exp2(S^T) converted to fp16
 //     is already the B-operand fragment of the second MFMA O^T = V^T P^T;
-//   * K and V tiles go global -> LDS directly (global_load_lds_dwordx4), double-buffered;
+//   * K and V tiles go global -> LDS directly (global_load_lds_dwordx4) into a 3-stage ring;
 //     V is kept [key][dim] in LDS and transposed on the way to registers with
 //     ds_read_b64_tr_b16; both tiles are XOR-swizzled against bank conflicts;
 //   * causal: tiles right of the diagonal are skipped, only tiles crossing it are masked.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace tfk {
 namespace {
 
-constexpr int kBM = 128;  // queries per workgroup
 constexpr int kBN = 64;   // keys per tile
-constexpr int kFaWaves = 4;
-constexpr int kFaThreads = kFaWaves * kWaveSize;
+constexpr int kStages = 3;
 
 // K tile [kBN][D]: 16 consecutive rows reading one logical chunk hit 16 bank groups.
 template <int CH>
@@ -62,10 +62,14 @@ TFK_DEVICE half4_t lds_read_tr4(const char* p) {
   return __builtin_bit_cast(half4_t, v);
 }
 
-template <int D, int DV, bool kVT, bool kCausal>
-__global__ __launch_bounds__(kFaThreads, 2) void flash_attention_fwd_kernel(
+// kWavesT wavefronts x 32 queries per workgroup.  8 wavefronts (256 queries) halve the
+// K/V traffic per query and put two wavefronts on every SIMD, so one wavefront's softmax
+// (VALU) overlaps the other's MFMAs; 4 wavefronts serve short query ranges.
+template <int D, int DV, bool kVT, bool kCausal, int kWavesT>
+__global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
     half_t* __restrict__ O, int Lq, int Lkv, float scale_log2, int q_tiles) {
+  constexpr int kBMq = kWavesT * 32;
   constexpr int kKChunks = D / 8;
   constexpr int kVChunks = kVT ? kBN / 8 : DV / 8;
   constexpr int kKBytes = kBN * D * 2;
@@ -73,84 +77,127 @@ __global__ __launch_bounds__(kFaThreads, 2) void flash_attention_fwd_kernel(
   constexpr int kStageBytes = kKBytes + kVBytes;
   constexpr int kNT = kBN / 32;
   constexpr int kDT = DV / 32;
+  constexpr int kKInstr = kKBytes / 1024;            // 1 KiB wavefront loads per K tile
+  constexpr int kVInstr = kVBytes / 1024;
+  constexpr int kKPerWave = (kKInstr + kWavesT - 1) / kWavesT;
+  constexpr int kVPerWave = (kVInstr + kWavesT - 1) / kWavesT;
+  constexpr int kLoadsPerTile = kKPerWave + kVPerWave;  // per wavefront (idle slots re-load)
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 31, lg = lane >> 5;
-  // heavy (late) query tiles first when causal
-  const int qt = kCausal ? (q_tiles - 1 - (int)blockIdx.x) : (int)blockIdx.x;
-  const size_t bh = blockIdx.y;
+  // Non-causal: x = query tile, y = slice.  Causal: x = slice, y = query tile with the heaviest
+  // (latest) tiles dispatched first across ALL slices, so the tail of the grid is made of the
+  // cheapest workgroups.
+  const int qt = kCausal ? (q_tiles - 1 - (int)blockIdx.y) : (int)blockIdx.x;
+  const size_t bh = kCausal ? blockIdx.x : blockIdx.y;
   Q += bh * (size_t)Lq * D;
   K += bh * (size_t)Lkv * D;
   V += bh * (size_t)Lkv * DV;
   O += bh * (size_t)Lq * DV;
 
-  const int q_row0 = qt * kBM + wave * 32;   // first query row of this wavefront
+  const int q_row0 = qt * kBMq + wave * 32;  // first query row of this wavefront
   const int m_row = q_row0 + lr;             // this lane's query row
   const int m_ld = min(m_row, Lq - 1);
 
+  // A negative scale is folded into Q (scores change sign, the scale becomes positive), so
+  // that the running maximum can be taken on raw scores and scaled once per row.
+  const float c = fmaxf(fabsf(scale_log2), 1e-30f);  // (a zero scale still yields uniform weights)
   half8_t qf[D / 16];
 #pragma unroll
-  for (int kk = 0; kk < D / 16; ++kk)
+  for (int kk = 0; kk < D / 16; ++kk) {
     qf[kk] = *reinterpret_cast<const half8_t*>(Q + (size_t)m_ld * D + kk * 16 + lg * 8);
+    if (scale_log2 < 0.f) qf[kk] = -qf[kk];
+  }
 
   int n_end = Lkv;
-  if (kCausal) n_end = min(Lkv, qt * kBM + kBM);
+  if (kCausal) n_end = min(Lkv, qt * kBMq + kBMq);
   const int num_tiles = (n_end + kBN - 1) / kBN;
 
-  auto issue_tile_loads = [&](int stage, int n0) {
-    char* sk = smem + stage * kStageBytes;
-    char* sv = sk + kKBytes;
-    {  // K tile: [kBN][D]
+  // ---- global -> LDS plan: wavefront instruction i of a tile covers 1 KiB of it ------------
+  const unsigned smem_base = lds_address(smem);
+  auto issue_tile_loads = [&](int tile) __attribute__((always_inline)) {
+    const int n0 = min(tile, num_tiles - 1) * kBN;  // clamped past the end (never read)
+    const unsigned sk = smem_base + (tile % kStages) * kStageBytes;
+    const unsigned sv = sk + kKBytes;
+#pragma unroll
+    for (int t = 0; t < kKPerWave; ++t) {  // K tile: [kBN][D]
+      const int i = (wave + kWavesT * t) % kKInstr;
       constexpr int kRowsPerInstr = 64 / kKChunks;
-      constexpr int kInstr = kBN * kKChunks / 64;
-      for (int i = wave; i < kInstr; i += kFaWaves) {
-        const int row = i * kRowsPerInstr + lane / kKChunks;
-        const int c = swz_k<kKChunks>(row, lane % kKChunks);
-        const int gr = min(n0 + row, Lkv - 1);
-        load_global_to_lds_16B(K + (size_t)gr * D + c * 8, sk + i * 1024);
-      }
+      const int row = i * kRowsPerInstr + lane / kKChunks;
+      const int cc = swz_k<kKChunks>(row, lane % kKChunks);
+      const int gr = min(n0 + row, Lkv - 1);
+      lds_dma_16B(K + (size_t)gr * D + cc * 8, sk + i * 1024);
     }
-    if constexpr (!kVT) {  // V tile: [kBN][DV]
+#pragma unroll
+    for (int t = 0; t < kVPerWave; ++t) {
+      const int i = (wave + kWavesT * t) % kVInstr;
       constexpr int kRowsPerInstr = 64 / kVChunks;
-      constexpr int kInstr = kBN * kVChunks / 64;
-      for (int i = wave; i < kInstr; i += kFaWaves) {
-        const int row = i * kRowsPerInstr + lane / kVChunks;
-        const int c = swz_v<kVChunks>(row, lane % kVChunks);
+      const int row = i * kRowsPerInstr + lane / kVChunks;
+      if constexpr (!kVT) {  // V tile: [kBN][DV]
+        const int cc = swz_v<kVChunks>(row, lane % kVChunks);
         const int gr = min(n0 + row, Lkv - 1);
-        load_global_to_lds_16B(V + (size_t)gr * DV + c * 8, sv + i * 1024);
-      }
-    } else {  // V^T tile: [DV][kBN] out of a [DV][Lkv] matrix
-      constexpr int kRowsPerInstr = 64 / kVChunks;
-      constexpr int kInstr = DV * kVChunks / 64;
-      for (int i = wave; i < kInstr; i += kFaWaves) {
-        const int row = i * kRowsPerInstr + lane / kVChunks;
-        const int c = swz_k<kVChunks>(row, lane % kVChunks);
-        const int gc = min(n0 + c * 8, Lkv - 8);
-        load_global_to_lds_16B(V + (size_t)row * Lkv + gc, sv + i * 1024);
+        lds_dma_16B(V + (size_t)gr * DV + cc * 8, sv + i * 1024);
+      } else {  // V^T tile: [DV][kBN] out of a [DV][Lkv] matrix
+        const int cc = swz_k<kVChunks>(row, lane % kVChunks);
+        const int gc = min(n0 + cc * 8, Lkv - 8);
+        lds_dma_16B(V + (size_t)row * Lkv + gc, sv + i * 1024);
       }
     }
   };
+
+  // ---- LDS -> register plan -----------------------------------------------------------------
+  // Every fragment read is (stage base) + (per-lane offset) + (compile-time immediate): the
+  // swizzles only XOR lane-dependent bits into the chunk index, so the lane part is computed
+  // once here and the tile loop spends no VALU on addresses beyond adding the stage base.
+  //   K fragment (nt, kk): row 32*nt + lr, logical chunk 2*kk + lg.
+  unsigned k_off[D / 16];
+#pragma unroll
+  for (int kk = 0; kk < D / 16; ++kk) k_off[kk] = lr * D * 2 + swz_k<kKChunks>(lr, 2 * kk + lg) * 16;
+  //   V fragment (dt, keys nk..nk+15), V kept [key][dim]: a 16-lane group transposes the 4 x 16
+  //   block of rows nk + 4*lg (+8) .. +3, columns 32*dt + 16*((lane>>4)&1) .. +15; lane r of the
+  //   group addresses row r/4, columns 4*(r%4) .. +3 of that block.
+  //   V^T fragment, V kept [dim][key]: row 32*dt + lr, keys nk + 4*lg (+8) .. +3.
+  constexpr int kVOffs = kVT ? 8 : kDT;
+  unsigned v_off[kVOffs];
+  if constexpr (!kVT) {
+    const int r16 = lane & 15;
+    const int row_l = 4 * lg + (r16 >> 2);
+    const int col_l = 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
+#pragma unroll
+    for (int dt = 0; dt < kDT; ++dt) {
+      const int col = dt * 32 + col_l;
+      v_off[dt] = row_l * DV * 2 + swz_v<kVChunks>(row_l, col / 8) * 16 + (col % 8) * 2;
+    }
+  } else {
+#pragma unroll
+    for (int cc = 0; cc < 8; ++cc) v_off[cc] = lr * kBN * 2 + swz_k<kVChunks>(lr, cc) * 16 + lg * 8;
+  }
 
   float16_t o_acc[kDT];
 #pragma unroll
   for (int dt = 0; dt < kDT; ++dt)
 #pragma unroll
     for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
-  float m_run = -INFINITY;  // running max of scale*log2(e)*score
+  float m_run = -INFINITY;  // reference max of the raw (sign-adjusted) scores (see below)
   float l_run = 0.f;        // this lane's share of the running sum
 
-  issue_tile_loads(0, 0);
-  wait_vmem_all();
-  __syncthreads();
+  // Ring of kStages tiles: tile it+kStages-1 is requested at the top of iteration it.
+#pragma unroll
+  for (int t = 0; t < kStages - 1; ++t) issue_tile_loads(t);
 
-  for (int it = 0; it < num_tiles; ++it) {
-    if (it + 1 < num_tiles) issue_tile_loads((it + 1) & 1, (it + 1) * kBN);
-    const char* sk = smem + (it & 1) * kStageBytes;
-    const char* sv = sk + kKBytes;
+  // Every iteration starts with the ring step: tile `it` has landed once only the younger
+  // tiles' loads are outstanding; the barrier also tells us every wavefront is done with
+  // tile it-1, whose stage is re-filled next.
+  auto ring_step = [&](int it) __attribute__((always_inline)) {
+    barrier_keep_vmem<(kStages - 2) * kLoadsPerTile>();
+    issue_tile_loads(it + kStages - 1);
+  };
+  auto process_tile = [&](int it, auto mask_c) __attribute__((always_inline)) {
+    constexpr bool kMask = decltype(mask_c)::value;
+    const unsigned stage_off = (it % kStages) * kStageBytes;
     const int n0 = it * kBN;
-
     // ---- S^T = K Q^T ------------------------------------------------------------------
     float16_t s[kNT];
 #pragma unroll
@@ -158,23 +205,18 @@ __global__ __launch_bounds__(kFaThreads, 2) void flash_attention_fwd_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[nt][r] = 0.f;
 #pragma unroll
-    for (int kk = 0; kk < D / 16; ++kk)
+    for (int kk = 0; kk < D / 16; ++kk) {
+      const char* kb = smem + (stage_off + k_off[kk]);
 #pragma unroll
       for (int nt = 0; nt < kNT; ++nt) {
-        const int row = nt * 32 + lr;
-        const half8_t kf = *reinterpret_cast<const half8_t*>(
-            sk + row * D * 2 + swz_k<kKChunks>(row, 2 * kk + lg) * 16);
+        const half8_t kf = *reinterpret_cast<const half8_t*>(kb + nt * 32 * D * 2);
         s[nt] = mfma_32x32x16(kf, qf[kk], s[nt]);
       }
+    }
 
-    // ---- scale, mask ------------------------------------------------------------------
+    // ---- mask -------------------------------------------------------------------------
     // s[nt][r] is the score of key n0 + 32*nt + 8*(r/4) + 4*lg + r%4 against query m_row
-    const bool need_mask = (kCausal && (n0 + kBN - 1 > q_row0)) || (n0 + kBN > Lkv);
-#pragma unroll
-    for (int nt = 0; nt < kNT; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[nt][r] *= scale_log2;
-    if (need_mask) {
+    if constexpr (kMask) {
 #pragma unroll
       for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
@@ -184,31 +226,44 @@ __global__ __launch_bounds__(kFaThreads, 2) void flash_attention_fwd_kernel(
         }
     }
 
-    // ---- online softmax ---------------------------------------------------------------
+    // ---- online softmax: p = exp2(c*s - c*m) -------------------------------------------
     float mx = s[0][0];
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nt][r]);
     mx = pair_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
+    // Lazy rescale: exponents are taken against a reference m_run that is only raised when a
+    // row's maximum has grown by more than kLazy (in log2 units) since the reference was set.
+    // Until then p = 2^(c*(s - m_run)) may reach 2^kLazy, which fp16 P and the fp32 sums hold
+    // easily, and the final O / l is unchanged because O and l share the reference.  Raising
+    // it costs a multiply of every O accumulator, so this skips it on almost every tile.
+    constexpr float kLazy = 8.f;
+    if (__builtin_amdgcn_ballot_w64((mx - m_run) * c > kLazy) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < kDT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+      m_run = m_new;
+    }
+    const float mc = m_run * c;
     float psum = 0.f;
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        s[nt][r] = __builtin_amdgcn_exp2f(s[nt][r] - m_new);
+        s[nt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][r], c, -mc));
         psum += s[nt][r];
       }
-    l_run = l_run * alpha + psum;
-#pragma unroll
-    for (int dt = 0; dt < kDT; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
+    l_run += psum;
 
     // ---- O^T += V^T P^T ---------------------------------------------------------------
+    const char* vb[kVOffs];
+#pragma unroll
+    for (int x = 0; x < kVOffs; ++x) vb[x] = smem + (stage_off + kKBytes + v_off[x]);
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
@@ -221,39 +276,45 @@ __global__ __launch_bounds__(kFaThreads, 2) void flash_attention_fwd_kernel(
         const int nk = nt * 32 + 16 * j;
 #pragma unroll
         for (int dt = 0; dt < kDT; ++dt) {
-          half8_t vf;
+          half4_t lo, hi;
           if constexpr (!kVT) {
-            const int r16 = lane & 15;
-            const int col = dt * 32 + 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
-            const int row_lo = nk + 4 * lg + (r16 >> 2);
-            const int row_hi = row_lo + 8;
-            const half4_t lo = lds_read_tr4(sv + row_lo * DV * 2 + swz_v<kVChunks>(row_lo, col / 8) * 16 + (col % 8) * 2);
-            const half4_t hi = lds_read_tr4(sv + row_hi * DV * 2 + swz_v<kVChunks>(row_hi, col / 8) * 16 + (col % 8) * 2);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              vf[t] = lo[t];
-              vf[4 + t] = hi[t];
-            }
+            lo = lds_read_tr4(vb[dt] + nk * DV * 2);
+            hi = lds_read_tr4(vb[dt] + (nk + 8) * DV * 2);
           } else {
-            const int row = dt * 32 + lr;
-            const int c0 = nk / 8;  // keys nk + 4*lg .. +3 live in chunk c0, half lg
-            const half4_t lo = *reinterpret_cast<const half4_t*>(
-                sv + row * kBN * 2 + swz_k<kVChunks>(row, c0) * 16 + lg * 8);
-            const half4_t hi = *reinterpret_cast<const half4_t*>(
-                sv + row * kBN * 2 + swz_k<kVChunks>(row, c0 + 1) * 16 + lg * 8);
+            lo = *reinterpret_cast<const half4_t*>(vb[nk / 8] + dt * 32 * kBN * 2);
+            hi = *reinterpret_cast<const half4_t*>(vb[nk / 8 + 1] + dt * 32 * kBN * 2);
+          }
+          half8_t vf;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-              vf[t] = lo[t];
-              vf[4 + t] = hi[t];
-            }
+          for (int t = 0; t < 4; ++t) {
+            vf[t] = lo[t];
+            vf[4 + t] = hi[t];
           }
           o_acc[dt] = mfma_32x32x16(vf, pb, o_acc[dt]);
         }
       }
+  };
 
-    wait_vmem_all();
-    __syncthreads();
+  // Tiles [0, n_plain) need no mask for this wavefront's 32 rows, [n_plain, n_compute) cross
+  // the diagonal or the end of the keys, and [n_compute, num_tiles) lie above the diagonal:
+  // the wavefront only keeps the ring (barrier + loads) going for its workgroup.
+  int n_plain = min(num_tiles, Lkv / kBN);
+  int n_compute = num_tiles;
+  if (kCausal) {
+    n_plain = max(0, min(n_plain, (q_row0 + 1) / kBN));
+    n_compute = min(num_tiles, (q_row0 + 31) / kBN + 1);
   }
+  int it = 0;
+  for (; it < n_plain; ++it) {
+    ring_step(it);
+    process_tile(it, std::false_type{});
+  }
+  for (; it < n_compute; ++it) {
+    ring_step(it);
+    process_tile(it, std::true_type{});
+  }
+  for (; it < num_tiles; ++it) ring_step(it);
+  wait_vmem_all();  // the clamped tail loads must not outlive the workgroup's LDS
 
   // ---- epilogue: O[m][d] = O^T[d][m] / l --------------------------------------------------
   const float l_tot = pair_sum(l_run);
@@ -271,21 +332,30 @@ __global__ __launch_bounds__(kFaThreads, 2) void flash_attention_fwd_kernel(
   }
 }
 
-template <int D, int DV, bool kVT, bool kCausal>
-int launch(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
-           float scale_log2, hipStream_t st) {
-  auto kern = flash_attention_fwd_kernel<D, DV, kVT, kCausal>;
-  constexpr int lds = 2 * (kBN * D * 2 + kBN * DV * 2);
+template <int D, int DV, bool kVT, bool kCausal, int kWavesT>
+int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
+             float scale_log2, hipStream_t st) {
+  auto kern = flash_attention_fwd_kernel<D, DV, kVT, kCausal, kWavesT>;
+  constexpr int lds = kStages * (kBN * D * 2 + kBN * DV * 2);
   static_assert(lds <= kMaxLdsBytes, "tiles do not fit in LDS");
   TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-  const int q_tiles = (Lq + kBM - 1) / kBM;
-  hipLaunchKernelGGL(kern, dim3(q_tiles, batch), dim3(kFaThreads), lds, st,
+  constexpr int bm = kWavesT * 32;
+  const int q_tiles = (Lq + bm - 1) / bm;
+  const dim3 grid = kCausal ? dim3(batch, q_tiles) : dim3(q_tiles, batch);
+  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * 64), lds, st,
                      static_cast<const half_t*>(Q), static_cast<const half_t*>(K),
                      static_cast<const half_t*>(V), static_cast<half_t*>(O), Lq, Lkv, scale_log2,
                      q_tiles);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
+}
+
+template <int D, int DV, bool kVT, bool kCausal>
+int launch(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
+           float scale_log2, hipStream_t st) {
+  if (Lq > 128) return launch_w<D, DV, kVT, kCausal, 8>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+  return launch_w<D, DV, kVT, kCausal, 4>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
 }
 
 template <int D, int DV>
@@ -312,7 +382,7 @@ extern "C" int tf_flash_attention_fwd_f16(const void* Q, const void* K, const vo
   TFK_REQUIRE(Q && K && V && O, TF_ERR_INVALID_ARG, "tf_flash_attention_fwd_f16: null pointer");
   TFK_REQUIRE(batch > 0 && Lq > 0 && Lkv > 0 && D > 0 && Dv > 0, TF_ERR_INVALID_ARG,
               "tf_flash_attention_fwd_f16: sizes must be positive");
-  TFK_REQUIRE(batch < 65536 && Lq < (1 << 24) && Lkv < (1 << 24), TF_ERR_INVALID_ARG,
+  TFK_REQUIRE(batch < 65536 && Lq < (1 << 21) && Lkv < (1 << 24), TF_ERR_INVALID_ARG,
               "tf_flash_attention_fwd_f16: dimension too large");
   TFK_REQUIRE(tile_length_q > 0 && tile_length_kv > 0 && tile_hidden_qk > 0 && tile_hidden_v > 0,
               TF_ERR_INVALID_ARG, "tf_flash_attention_fwd_f16: tile sizes must be positive");
