@@ -1,0 +1,325 @@
+// GPU test kernels for the tile-programming headers, exported with a C ABI so the pytest
+// files can drive them through ctypes.  They restate the asserted tests of the reference
+// (tests/cpp/cell/test_g2s_load.cu, test_s2r_copy.cu, test_swizzled_copy.cu, test_gemm.cu) and
+// add asserted tests for what the reference only prints (G2R/R2G, reduce, broadcast, mask).
+#include <hip/hip_runtime.h>
+
+#include "cell/mod.hpp"
+#include "kernels/gemm_device.hpp"
+#include "types/mod.hpp"
+
+using namespace tilefusion;
+using namespace tilefusion::cell;
+using namespace tilefusion::cell::copy;
+namespace tl = tile_layout;
+
+#define TT_API extern "C" __attribute__((visibility("default")))
+
+static int launch_status() {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return (int)e;
+  return (int)hipDeviceSynchronize();
+}
+
+// ---- 1. global -> LDS -> global round trip (test_g2s_load.cu:19-45,144-268) ------------------
+template <typename Element, typename WarpLayout, typename Layout, bool kSwizzled, int kBytes>
+__global__ void k_g2s_roundtrip(const Element* in, Element* out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char buf[];
+  using Global = GlobalTile<Element, Layout>;
+  using Shared = SharedTile<Element, Layout, kSwizzled, kBytes>;
+  Global g_in(in), g_out(out);
+  Shared s(reinterpret_cast<Element*>(buf));
+  GlobalToSharedLoader<Shared, WarpLayout> load;
+  SharedToGlobalStorer<Shared, WarpLayout> store;
+  load(g_in, s);
+  __copy_async();
+  __syncthreads();
+  store(s, g_out);
+}
+template <typename Element, typename WarpLayout, typename Layout, bool kSwizzled, int kBytes>
+static int run_g2s(const void* in, void* out) {
+  hipLaunchKernelGGL((k_g2s_roundtrip<Element, WarpLayout, Layout, kSwizzled, kBytes>), dim3(1),
+                     dim3(tl::get_numel<WarpLayout> * WARP_SIZE), Layout::kNumel * sizeof(Element), 0,
+                     static_cast<const Element*>(in), static_cast<Element*>(out));
+  return launch_status();
+}
+TT_API int tt_g2s_roundtrip(int variant, const void* in, void* out) {
+  switch (variant) {
+    case 0: return run_g2s<__half, tl::RowMajor<1, 1>, tl::RowMajor<16, 64>, false, 128>(in, out);
+    case 1: return run_g2s<__half, tl::RowMajor<1, 1>, tl::RowMajor<64, 64>, true, 128>(in, out);
+    case 2: return run_g2s<__half, tl::RowMajor<2, 2>, tl::RowMajor<128, 128>, true, 128>(in, out);
+    case 3: return run_g2s<__half, tl::RowMajor<2, 2>, tl::RowMajor<128, 128>, true, 64>(in, out);
+    case 4: return run_g2s<__half, tl::RowMajor<4, 2>, tl::RowMajor<128, 256>, true, 64>(in, out);
+    case 5: return run_g2s<__half, tl::RowMajor<2, 1>, tl::ColMajor<64, 64>, true, 128>(in, out);
+    case 6: return run_g2s<__half, tl::RowMajor<2, 2>, tl::ColMajor<128, 64>, true, 64>(in, out);
+    case 7: return run_g2s<float, tl::RowMajor<2, 2>, tl::RowMajor<64, 64>, true, 128>(in, out);
+    case 8: return run_g2s<float, tl::RowMajor<1, 1>, tl::ColMajor<32, 32>, true, 64>(in, out);
+    case 9: return run_g2s<__half, tl::RowMajor<1, 4>, tl::RowMajor<32, 256>, false, 128>(in, out);
+    default: return -1;
+  }
+}
+TT_API void tt_g2s_shape(int variant, int* rows, int* cols, int* elem_bytes, int* col_major) {
+  static const int t[10][4] = {{16, 64, 2, 0}, {64, 64, 2, 0}, {128, 128, 2, 0}, {128, 128, 2, 0}, {128, 256, 2, 0},
+                               {64, 64, 2, 1}, {128, 64, 2, 1}, {64, 64, 4, 0}, {32, 32, 4, 1}, {32, 256, 2, 0}};
+  *rows = t[variant][0]; *cols = t[variant][1]; *elem_bytes = t[variant][2]; *col_major = t[variant][3];
+}
+
+// ---- 2. swizzled and plain LDS tiles give identical register fragments, and an accumulator
+//         tile survives register -> LDS -> global (test_swizzled_copy.cu:27-94, test_s2r_copy.cu) --
+template <typename WarpLayout, int kRows, int kCols, int kChunk, int kBytes>
+__global__ void k_swizzled_fragments(const __half* a_in, const __half* b_in, int* mismatches) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char buf[];
+  __half* base = reinterpret_cast<__half*>(buf);
+  using GlobalA = GlobalTile<__half, tl::RowMajor<kRows, kCols>>;
+  using GlobalB = GlobalTile<__half, tl::ColMajor<kCols, kRows>>;
+  using SA0 = SharedTile<__half, tl::RowMajor<kRows, kCols>, false, kBytes>;
+  using SA1 = SharedTile<__half, tl::RowMajor<kRows, kCols>, true, kBytes>;
+  using SB0 = SharedTile<__half, tl::ColMajor<kCols, kRows>, false, kBytes>;
+  using SB1 = SharedTile<__half, tl::ColMajor<kCols, kRows>, true, kBytes>;
+  SA0 sa0(base);
+  SA1 sa1(base + kRows * kCols);
+  SB0 sb0(base + 2 * kRows * kCols);
+  SB1 sb1(base + 3 * kRows * kCols);
+  GlobalA ga(a_in);
+  GlobalB gb(b_in);
+  { GlobalToSharedLoader<SA0, WarpLayout> l; l(ga, sa0); }
+  { GlobalToSharedLoader<SA1, WarpLayout> l; l(ga, sa1); }
+  { GlobalToSharedLoader<SB0, WarpLayout> l; l(gb, sb0); }
+  { GlobalToSharedLoader<SB1, WarpLayout> l; l(gb, sb1); }
+  __copy_async();
+  __syncthreads();
+  constexpr int kWR = tl::num_rows<WarpLayout>, kWC = tl::num_cols<WarpLayout>;
+  using RegA = RegTile<BaseTileRowMajor<__half>, tl::RowMajor<kRows / kWR / 16, kChunk / 32>>;
+  using RegB = RegTile<BaseTileColMajor<__half>, tl::ColMajor<kChunk / 32, kRows / kWC / 16>>;
+  using IterA0 = STileIterator<SA0, TileShape<kRows, kChunk>>;
+  using IterA1 = STileIterator<SA1, TileShape<kRows, kChunk>>;
+  using IterB0 = STileIterator<SB0, TileShape<kChunk, kRows>>;
+  using IterB1 = STileIterator<SB1, TileShape<kChunk, kRows>>;
+  IterA0 ia0(base);
+  IterA1 ia1(base + kRows * kCols);
+  IterB0 ib0(base + 2 * kRows * kCols);
+  IterB1 ib1(base + 3 * kRows * kCols);
+  SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont> la;
+  SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont> lb;
+  int bad = 0;
+  for (int k = 0; k < IterA0::sc1; ++k) {
+    RegA ra0, ra1;
+    RegB rb0, rb1;
+    la(ia0(k), ra0);
+    la(ia1(k), ra1);
+    lb(ib0(k), rb0);
+    lb(ib1(k), rb1);
+    const __half* p0 = ra0.data()[0].data();
+    const __half* p1 = ra1.data()[0].data();
+    for (int e = 0; e < RegA::kNumel * 8; ++e) bad += (__half2float(p0[e]) != __half2float(p1[e]));
+    const __half* q0 = rb0.data()[0].data();
+    const __half* q1 = rb1.data()[0].data();
+    for (int e = 0; e < RegB::kNumel * 8; ++e) bad += (__half2float(q0[e]) != __half2float(q1[e]));
+    // and the fragment really is the documented block of the source: element 0 of base tile (0,0)
+    const int lane = threadIdx.x % WARP_SIZE;
+    const int wr = warp::warp_row_id<WarpLayout>();
+    const float want = __half2float(a_in[(wr * (kRows / kWR) + lane % 16) * kCols + k * kChunk + 8 * (lane / 16)]);
+    bad += (__half2float(p0[0]) != want);
+  }
+  if (bad) atomicAdd(mismatches, bad);
+}
+TT_API int tt_swizzled_fragments(int variant, const void* a, const void* b, int* mismatches) {
+  const __half* pa = static_cast<const __half*>(a);
+  const __half* pb = static_cast<const __half*>(b);
+  switch (variant) {
+    case 0:
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<1, 1>, 64, 64, 32, 128>), dim3(1), dim3(64), 4 * 64 * 64 * 2, 0, pa, pb, mismatches);
+      break;
+    case 1:
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<2, 2>, 128, 128, 64, 128>), dim3(1), dim3(256), 4 * 128 * 128 * 2, 0, pa, pb, mismatches);
+      break;
+    case 2:
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<2, 2>, 64, 128, 32, 64>), dim3(1), dim3(256), 4 * 64 * 128 * 2, 0, pa, pb, mismatches);
+      break;
+    case 3:
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<4, 1>, 64, 64, 64, 64>), dim3(1), dim3(256), 4 * 64 * 64 * 2, 0, pa, pb, mismatches);
+      break;
+    default: return -1;
+  }
+  return launch_status();
+}
+
+template <typename WarpLayout, int kRows, int kCols>
+__global__ void k_acc_roundtrip(const float* in, float* out_direct, float* out_via_lds, __half* out_half) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char buf[];
+  constexpr int kWR = tl::num_rows<WarpLayout>, kWC = tl::num_cols<WarpLayout>;
+  using Global = GlobalTile<float, tl::RowMajor<kRows, kCols>>;
+  using GlobalH = GlobalTile<__half, tl::RowMajor<kRows, kCols>>;
+  using Reg = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kRows / kWR / 16, kCols / kWC / 16>>;
+  using RegH = RegTile<BaseTileAccRowMajor<__half>, tl::RowMajor<kRows / kWR / 16, kCols / kWC / 16>>;
+  using Shared = SharedTile<float, tl::RowMajor<kRows, kCols>, true, 128>;
+  Global g_in(in), g_direct(out_direct), g_lds(out_via_lds);
+  GlobalH g_half(out_half);
+  Shared s(reinterpret_cast<float*>(buf));
+  Reg r;
+  GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+  g2r(g_in, r);
+  RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+  r2g(r, g_direct);
+  RegToSharedStorer<Reg, WarpLayout> r2s;
+  r2s(r, s);
+  __syncthreads();
+  SharedToGlobalStorer<Shared, WarpLayout> s2g;
+  s2g(s, g_lds);
+  RegH rh;
+  compute::RegTileConvert<Reg, RegH> cast;
+  cast(r, rh);
+  RegToGlobalStorer<GlobalH, RegH, WarpLayout> r2gh;
+  r2gh(rh, g_half);
+}
+TT_API int tt_acc_roundtrip(int variant, const void* in, void* out_direct, void* out_lds, void* out_half) {
+  const float* pi = static_cast<const float*>(in);
+  float* po = static_cast<float*>(out_direct);
+  float* pl = static_cast<float*>(out_lds);
+  __half* ph = static_cast<__half*>(out_half);
+  switch (variant) {
+    case 0:
+      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<1, 1>, 32, 64>), dim3(1), dim3(64), 32 * 64 * 4, 0, pi, po, pl, ph);
+      break;
+    case 1:
+      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<2, 2>, 128, 64>), dim3(1), dim3(256), 128 * 64 * 4, 0, pi, po, pl, ph);
+      break;
+    default: return -1;
+  }
+  return launch_status();
+}
+
+// ---- 3. the README example: GEMM with global -> register loaders only (README.md:56-112,
+//         examples/101_gemm/01_gemm_global_reg/gemm.hpp:62-95) with the consistent tile shapes ----
+namespace readme {
+using InType = __half;
+using AccType = float;
+using WarpLayout = tl::RowMajor<2, 2>;
+constexpr int kM = 128, kN = 64, kK = 256, kTK = 32;
+using GlobalA = GlobalTile<InType, tl::RowMajor<kM, kK>>;
+using IteratorA = TileIterator<GlobalA, TileShape<kM, kTK>>;
+using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kM / 2 / 16, kTK / 32>>;
+using ALoader = GlobalToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kN>>;
+using IteratorB = TileIterator<GlobalB, TileShape<kTK, kN>>;
+using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kN / 2 / 16>>;
+using BLoader = GlobalToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+using GlobalC = GlobalTile<AccType, tl::RowMajor<kM, kN>>;
+using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kM / 2 / 16, kN / 2 / 16>>;
+using CStorer = RegToGlobalStorer<GlobalC, RegC, WarpLayout>;
+
+__global__ void simple_gemm(const InType* dA, const InType* dB, AccType* dC) {
+  IteratorA gAs(dA);
+  RegA rA;
+  ALoader loader_a;
+  IteratorB gBs(dB);
+  RegB rB;
+  BLoader loader_b;
+  RegC acc;
+  GlobalC gC(dC);
+  CStorer storer_c;
+  for (int k = 0; k < IteratorA::sc1; ++k) {
+    loader_a(gAs(k), rA);
+    loader_b(gBs(k), rB);
+    __syncthreads();
+    compute::gemm(rA, rB, acc);
+  }
+  __syncthreads();
+  storer_c(acc, gC);
+}
+}  // namespace readme
+TT_API int tt_readme_gemm(const void* a, const void* b, void* c) {
+  hipLaunchKernelGGL(readme::simple_gemm, dim3(1), dim3(tl::get_numel<readme::WarpLayout> * WARP_SIZE), 0, 0,
+                     static_cast<const __half*>(a), static_cast<const __half*>(b), static_cast<float*>(c));
+  return launch_status();
+}
+
+// ---- 4. ke_gemm composed from the primitives (test_gemm.cu:172-215,316-375) ------------------
+template <typename Traits, typename AccType>
+__global__ void k_ke_gemm(const __half* a, const __half* b, AccType* c) {
+  kernels::ke_gemm<__half, AccType, Traits>(a, b, c);
+}
+template <typename WarpLayout, typename AccType, int M, int N, int K, int TM, int TN, int TK, int RK, int Stages, int Bytes>
+static int run_ke_gemm(const void* a, const void* b, void* c) {
+  using Traits = kernels::KeGemmTraits<__half, AccType, WarpLayout, M, N, K, TM, TN, TK, RK, Stages, Bytes>;
+  auto kern = k_ke_gemm<Traits, AccType>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Traits::kSharedBytes) != hipSuccess) return -2;
+  hipLaunchKernelGGL(kern, dim3(M / TM, N / TN), dim3(Traits::kThreads), Traits::kSharedBytes, 0,
+                     static_cast<const __half*>(a), static_cast<const __half*>(b), static_cast<AccType*>(c));
+  return launch_status();
+}
+TT_API int tt_ke_gemm(int variant, const void* a, const void* b, void* c) {
+  switch (variant) {
+    case 0: return run_ke_gemm<tl::RowMajor<1, 1>, float, 64, 64, 64, 64, 64, 64, 16, 1, 64>(a, b, c);
+    case 1: return run_ke_gemm<tl::RowMajor<1, 1>, float, 128, 128, 128, 64, 64, 64, 16, 1, 64>(a, b, c);
+    case 2: return run_ke_gemm<tl::RowMajor<2, 2>, float, 256, 256, 256, 128, 128, 64, 32, 2, 128>(a, b, c);
+    case 3: return run_ke_gemm<tl::RowMajor<2, 2>, __half, 256, 128, 512, 64, 128, 128, 32, 2, 64>(a, b, c);
+    case 4: return run_ke_gemm<tl::RowMajor<4, 1>, float, 128, 64, 256, 128, 64, 32, 32, 3, 64>(a, b, c);
+    case 5: return run_ke_gemm<tl::RowMajor<2, 4>, float, 512, 512, 128, 128, 256, 64, 64, 2, 128>(a, b, c);
+    default: return -1;
+  }
+}
+TT_API void tt_ke_gemm_shape(int variant, int* m, int* n, int* k, int* c_is_half) {
+  static const int t[6][4] = {{64, 64, 64, 0}, {128, 128, 128, 0}, {256, 256, 256, 0}, {256, 128, 512, 1}, {128, 64, 256, 0}, {512, 512, 128, 0}};
+  *m = t[variant][0]; *n = t[variant][1]; *k = t[variant][2]; *c_is_half = t[variant][3];
+}
+
+// ---- 5. reduce / broadcast / map / mask on an accumulator tile (print-only in the reference:
+//         tests/cpp/cell/test_reduce.cu, test_broadcast.cu, test_flash_attn.cu) ------------------
+template <typename WarpLayout, int kRows, int kCols>
+__global__ void k_softmax_pieces(const float* in, float* row_max, float* row_sum, float* out, int row_offset,
+                                 int col_offset) {
+  constexpr int kWR = tl::num_rows<WarpLayout>;
+  static_assert(tl::num_cols<WarpLayout> == 1, "rows must not be split across wavefronts");
+  using Global = GlobalTile<float, tl::RowMajor<kRows, kCols>>;
+  using Reg = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kRows / kWR / 16, kCols / 16>>;
+  using Vec = RegTile<float, tl::RowMajor<Reg::kRows, 4>>;
+  Global g_in(in), g_out(out);
+  Reg t;
+  GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+  g2r(g_in, t);
+  ApplyMask<Reg, WarpLayout, BaseTileShape<float>, MaskMode::kCausal> mask;
+  mask(t, row_offset, col_offset, -INFINITY);
+  Vec vmax, vsum;
+  compute::MaxReduce<Reg, tl::Layout::kRowMajor> rmax;
+  rmax(t, vmax);
+  compute::BroadcastSub<Vec, Reg, tl::Layout::kRowMajor> bsub;
+  bsub(vmax, t);
+  compute::RegTileExp<Reg> rexp;
+  rexp(t, t);
+  compute::SumReduce<Reg, tl::Layout::kRowMajor> rsum;
+  rsum(t, vsum);
+  compute::BroadcastDiv<Vec, Reg, tl::Layout::kRowMajor> bdiv;
+  bdiv(vsum, t);
+  compute::BroadcastScalarMul<Reg> smul;
+  smul(t, 2.0f, t);
+  RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+  r2g(t, g_out);
+  const int lane = threadIdx.x % WARP_SIZE;
+  const int wrow = warp::warp_row_id<WarpLayout>() * (kRows / kWR);
+  if (lane % 16 == 0) {
+    for (int i = 0; i < Reg::kRows; ++i)
+      for (int r = 0; r < 4; ++r) {
+        row_max[wrow + 16 * i + 4 * (lane / 16) + r] = vmax(i, r);
+        row_sum[wrow + 16 * i + 4 * (lane / 16) + r] = vsum(i, r);
+      }
+  }
+}
+TT_API int tt_softmax_pieces(int variant, const void* in, void* row_max, void* row_sum, void* out, int row_offset,
+                             int col_offset) {
+  const float* pi = static_cast<const float*>(in);
+  float *pm = static_cast<float*>(row_max), *ps = static_cast<float*>(row_sum), *po = static_cast<float*>(out);
+  switch (variant) {
+    case 0:
+      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<1, 1>, 16, 16>), dim3(1), dim3(64), 0, 0, pi, pm, ps, po, row_offset, col_offset);
+      break;
+    case 1:
+      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<1, 1>, 32, 64>), dim3(1), dim3(64), 0, 0, pi, pm, ps, po, row_offset, col_offset);
+      break;
+    case 2:
+      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<4, 1>, 128, 128>), dim3(1), dim3(256), 0, 0, pi, pm, ps, po, row_offset, col_offset);
+      break;
+    default: return -1;
+  }
+  return launch_status();
+}

@@ -1,0 +1,85 @@
+// Broadcast of a reduced vector (or a scalar) over an accumulator register tile (counterpart
+// of include/cell/compute/broadcast.hpp:14-187).  Row-major: src is the kRows x 4 vector that
+// SumReduce / MaxReduce produce and element (i, r) meets all columns of tile row
+// 16*i + 4*(l/16) + r.  The fused forms compute dst = f(dst, src) in place.
+#pragma once
+
+#include "cell/compute/math_functor.hpp"
+#include "types/register.hpp"
+
+namespace tilefusion::cell::compute {
+namespace tl = tile_layout;
+
+template <typename SrcTile, typename DstTile, tl::Layout kLayout>
+struct Broadcast {
+  using DType = typename DstTile::DType::DType;
+  static constexpr int kRows = DstTile::kRows, kCols = DstTile::kCols;
+  DEVICE void operator()(const SrcTile& src, DstTile& dst) {
+#pragma unroll
+    for (int i = 0; i < kRows; ++i)
+#pragma unroll
+      for (int j = 0; j < kCols; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if constexpr (kLayout == tl::Layout::kRowMajor) {
+            dst(i, j)(r, 0) = src(i, r);
+          } else {
+            dst(i, j)(0, r) = src(r, j);
+          }
+        }
+  }
+};
+
+template <typename SrcTile, typename DstTile, typename Functor, tl::Layout kLayout>
+struct BroadcastFuse {
+  using DType = typename DstTile::DType::DType;
+  static constexpr int kRows = DstTile::kRows, kCols = DstTile::kCols;
+  DEVICE void operator()(const SrcTile& src, DstTile& dst) {
+    Functor f;
+#pragma unroll
+    for (int i = 0; i < kRows; ++i)
+#pragma unroll
+      for (int j = 0; j < kCols; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if constexpr (kLayout == tl::Layout::kRowMajor) {
+            f(dst(i, j)(r, 0), src(i, r), dst(i, j)(r, 0));
+          } else {
+            f(dst(i, j)(0, r), src(r, j), dst(i, j)(0, r));
+          }
+        }
+  }
+};
+
+// dst = f(src, scalar) element-wise, on a base tile or on a tile of base tiles
+template <typename RegTile, typename Functor>
+struct BroadcastScalar {
+  template <typename Element>
+  DEVICE void operator()(const RegTile& src, Element scalar, RegTile& dst) {
+    if constexpr (requires(const typename RegTile::DType& d) { d.data(); }) {
+      BroadcastScalar<typename RegTile::DType, Functor> inner;
+#pragma unroll
+      for (int i = 0; i < RegTile::kNumel; ++i) inner(src.data()[i], scalar, dst.mutable_data()[i]);
+    } else {
+      Functor f;
+#pragma unroll
+      for (int i = 0; i < RegTile::kNumel; ++i) f(src.data()[i], scalar, dst.mutable_data()[i]);
+    }
+  }
+};
+
+template <typename SrcTile, typename DstTile, tl::Layout kLayout>
+using BroadcastAdd = BroadcastFuse<SrcTile, DstTile, Add<typename DstTile::DType::DType>, kLayout>;
+template <typename SrcTile, typename DstTile, tl::Layout kLayout>
+using BroadcastSub = BroadcastFuse<SrcTile, DstTile, Sub<typename DstTile::DType::DType>, kLayout>;
+template <typename SrcTile, typename DstTile, tl::Layout kLayout>
+using BroadcastMul = BroadcastFuse<SrcTile, DstTile, Mul<typename DstTile::DType::DType>, kLayout>;
+template <typename SrcTile, typename DstTile, tl::Layout kLayout>
+using BroadcastDiv = BroadcastFuse<SrcTile, DstTile, Div<typename DstTile::DType::DType>, kLayout>;
+
+template <typename RegTile>
+using BaseBroadcastScalarMul = BroadcastScalar<RegTile, Mul<typename RegTile::DType>>;
+template <typename RegTile>
+using BroadcastScalarMul = BroadcastScalar<RegTile, Mul<typename RegTile::DType::DType>>;
+
+}  // namespace tilefusion::cell::compute

@@ -1,0 +1,174 @@
+// GEMM macro kernel composed from the tile primitives (counterpart of
+// include/kernels/gemm_device.cuh:16-419): C[M,N] = A[M,K] * B[K,N], A row-major, B column-major,
+// one workgroup per [kTM, kTN] tile of C, K walked in kTK chunks through LDS and in kRK steps
+// through registers.
+//
+// This is the portable, shape-generic form of the kernel - every shape is a template
+// parameter and any kernel written against the tile API composes the same way.  The library's
+// own tuned GEMM entry point (tf_gemm_f16) is a separate hand-scheduled kernel.
+//
+// Differences from the reference that follow from the hardware: a wavefront has 64 lanes
+// (kThreads = |WarpLayout| * 64), the MFMA reduces 32 values of k per instruction (kRK is
+// rounded up to a multiple of 32), and with kNumStages >= 2 the next k-chunk is fetched into a
+// second LDS buffer while the current one is multiplied (the reference's level-1 pipeline).
+#pragma once
+
+#include "cell/mod.hpp"
+#include "types/mod.hpp"
+
+namespace tilefusion::kernels {
+using namespace tilefusion::cell;
+using namespace tilefusion::cell::copy;
+namespace tl = tile_layout;
+
+template <typename InType_, typename AccType_, typename WarpLayout_, int kM_, int kN_, int kK_, int kTM_,
+          int kTN_, int kTK_, int kRK_, int kNumStages_, int kSharedAccess = 64>
+struct KeGemmTraits {
+  using InType = InType_;
+  using AccType = AccType_;
+  using WarpLayout = WarpLayout_;
+  using BaseShape = BaseTileShape<InType>;  // 16 x 32 operand block
+  static constexpr int kNumStages = kNumStages_;
+
+  static constexpr int kThreads = tl::get_numel<WarpLayout> * WARP_SIZE;
+  static constexpr int kWarpPerRow = tl::num_rows<WarpLayout>;
+  static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
+
+  static constexpr int kM = kM_, kN = kN_, kK = kK_;
+  static constexpr int kTM = kTM_, kTN = kTN_, kTK = kTK_;
+  static constexpr int kRK = kRK_ < BaseShape::kCols ? BaseShape::kCols : kRK_;
+  static_assert(kTK % kRK == 0 && kRK % BaseShape::kCols == 0, "kTK must be a multiple of kRK (a multiple of 32)");
+  static constexpr bool kSwizzled = true;
+
+  using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK, kK>>;
+  using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
+  using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, kSwizzled, kSharedAccess>;
+  using SIteratorA = STileIterator<SharedA, TileShape<kTM, kRK>>;
+  static constexpr int kAMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kAKs = kRK / BaseShape::kCols;
+  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAMs, kAKs>>;
+  using G2SLoaderA = GlobalToSharedLoader<SharedA, WarpLayout>;
+  using S2RLoaderA = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
+
+  using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kTN, kK>>;
+  using GIteratorB = GTileIterator<GlobalB, TileShape<kTK, kTN>>;
+  using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, kSwizzled, kSharedAccess>;
+  using SIteratorB = STileIterator<SharedB, TileShape<kRK, kTN>>;
+  static_assert(GIteratorA::sc1 == GIteratorB::sc0 && SIteratorA::sc1 == SIteratorB::sc0, "mismatched K dimension");
+  static constexpr int kBKs = kRK / BaseShape::kCols;                   // 32 values of k per base tile
+  static constexpr int kBNs = kTN / kWarpPerCol / BaseShape::kRows;     // 16 columns per base tile
+  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kBKs, kBNs>>;
+  using G2SLoaderB = GlobalToSharedLoader<SharedB, WarpLayout>;
+  using S2RLoaderB = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
+
+  using GlobalC = GlobalTile<AccType, tl::RowMajor<kTM, kTN, kN>>;
+  using SharedC = SharedTile<AccType, tl::RowMajor<kTM, kTN>, false>;
+  static constexpr int kCMs = kTM / kWarpPerRow / 16;
+  static constexpr int kCNs = kTN / kWarpPerCol / 16;
+  using RegC = RegTile<BaseTileAccRowMajor<AccType>, tl::RowMajor<kCMs, kCNs>>;
+  using RegAcc = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kCMs, kCNs>>;
+  using R2GStorerC = RegToGlobalStorer<GlobalC, RegC, WarpLayout>;
+  using R2SStorerC = RegToSharedStorer<RegC, WarpLayout>;
+  using S2GStorerC = SharedToGlobalStorer<SharedC, WarpLayout>;
+
+  static constexpr int kStageElems = SharedA::kNumel + SharedB::kNumel;
+  static constexpr int kLdsStages = kNumStages >= 2 ? 2 : 1;
+  static constexpr int kSharedBytes = kStageElems * kLdsStages * (int)sizeof(InType);
+};
+
+namespace detail {
+template <typename KeTraits, typename InType, typename AccType>
+DEVICE void store_acc(const typename KeTraits::RegAcc& acc, AccType* dC) {
+  typename KeTraits::GlobalC gC(dC);
+  typename KeTraits::R2GStorerC r2g;
+  if constexpr (std::is_same_v<AccType, float>) {
+    r2g(acc, gC);
+  } else {
+    typename KeTraits::RegC out;
+    compute::RegTileConvert<typename KeTraits::RegAcc, typename KeTraits::RegC> cast;
+    cast(acc, out);
+    r2g(out, gC);
+  }
+}
+}  // namespace detail
+
+// kNumStages == 1: load chunk, synchronise, multiply.  kNumStages >= 2: double-buffered LDS.
+template <typename InType, typename AccType, typename KeTraits>
+DEVICE void ke_gemm(const InType* dA, const InType* dB, AccType* dC) {
+  constexpr int kN = KeTraits::kN, kK = KeTraits::kK, kTM = KeTraits::kTM, kTN = KeTraits::kTN;
+  const InType* gA_ptr = dA + ptrdiff_t(blockIdx.x) * kTM * kK;
+  const InType* gB_ptr = dB + ptrdiff_t(blockIdx.y) * kTN * kK;
+  AccType* gC_ptr = dC + ptrdiff_t(blockIdx.x) * kTM * kN + ptrdiff_t(blockIdx.y) * kTN;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char tilefusion_lds[];
+  InType* lds = reinterpret_cast<InType*>(tilefusion_lds);
+
+  typename KeTraits::GIteratorA gAs(gA_ptr);
+  typename KeTraits::GIteratorB gBs(gB_ptr);
+  typename KeTraits::RegA rA;
+  typename KeTraits::RegB rB;
+  typename KeTraits::RegAcc acc;
+  typename KeTraits::G2SLoaderA g2s_a;
+  typename KeTraits::G2SLoaderB g2s_b;
+  typename KeTraits::S2RLoaderA s2r_a;
+  typename KeTraits::S2RLoaderB s2r_b;
+
+  constexpr int kChunks = KeTraits::GIteratorA::sc1;
+  constexpr int kStages = KeTraits::kLdsStages;
+  auto stage_a = [&](int s) { return typename KeTraits::SharedA(lds + s * KeTraits::kStageElems); };
+  auto stage_b = [&](int s) {
+    return typename KeTraits::SharedB(lds + s * KeTraits::kStageElems + KeTraits::SharedA::kNumel);
+  };
+
+  if constexpr (kStages == 2) {
+    auto sA0 = stage_a(0);
+    auto sB0 = stage_b(0);
+    g2s_a(gAs(0), sA0);
+    g2s_b(gBs(0), sB0);
+    __copy_async();
+    __syncthreads();
+  }
+  for (int k1 = 0; k1 < kChunks; ++k1) {
+    const int cur = kStages == 2 ? (k1 & 1) : 0;
+    if constexpr (kStages == 2) {
+      if (k1 + 1 < kChunks) {
+        auto sAn = stage_a(cur ^ 1);
+        auto sBn = stage_b(cur ^ 1);
+        g2s_a(gAs(k1 + 1), sAn);
+        g2s_b(gBs(k1 + 1), sBn);
+      }
+    } else {
+      auto sA0 = stage_a(0);
+      auto sB0 = stage_b(0);
+      g2s_a(gAs(k1), sA0);
+      g2s_b(gBs(k1), sB0);
+      __copy_async();
+      __syncthreads();
+    }
+    typename KeTraits::SIteratorA sAs(lds + cur * KeTraits::kStageElems);
+    typename KeTraits::SIteratorB sBs(lds + cur * KeTraits::kStageElems + KeTraits::SharedA::kNumel);
+#pragma unroll
+    for (int k2 = 0; k2 < KeTraits::SIteratorA::sc1; ++k2) {
+      s2r_a(sAs(k2), rA);
+      s2r_b(sBs(k2), rB);
+      compute::gemm(rA, rB, acc);
+    }
+    __copy_async();
+    __syncthreads();
+  }
+  detail::store_acc<KeTraits, InType, AccType>(acc, gC_ptr);
+}
+
+// The reference's level-1 / level-2 pipelines are what kNumStages >= 2 selects here.
+template <typename InType, typename AccType, typename KeTraits>
+DEVICE void ke_gemm_level1_pipeline(const InType* dA, const InType* dB, AccType* dC) {
+  static_assert(KeTraits::kNumStages >= 2, "the pipelined kernels need kNumStages >= 2");
+  ke_gemm<InType, AccType, KeTraits>(dA, dB, dC);
+}
+template <typename InType, typename AccType, typename KeTraits>
+DEVICE void ke_gemm_level2_pipeline(const InType* dA, const InType* dB, AccType* dC) {
+  static_assert(KeTraits::kNumStages >= 2, "the pipelined kernels need kNumStages >= 2");
+  ke_gemm<InType, AccType, KeTraits>(dA, dB, dC);
+}
+
+}  // namespace tilefusion::kernels
