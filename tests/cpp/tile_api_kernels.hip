@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 
 #include "cell/mod.hpp"
+#include "kernels/flash_attention_device.hpp"
+#include "kernels/fused_two_gemms_device.hpp"
 #include "kernels/gemm_device.hpp"
 #include "types/mod.hpp"
 
@@ -322,4 +324,72 @@ TT_API int tt_softmax_pieces(int variant, const void* in, void* row_max, void* r
     default: return -1;
   }
   return launch_status();
+}
+
+// ---- 6. fused back-to-back GEMM composed from the primitives (tests/python/test_fused_two_gemms.py:
+//         M, N, K, P = 256, 128, 64, 64 with 64-wide tiles) ------------------------------------------
+template <typename Traits>
+__global__ void k_ke_fused(const __half* a, const __half* b, const __half* c, __half* d) {
+  kernels::ke_fused_two_gemms<__half, float, Traits>(a, b, c, d);
+}
+template <typename WarpLayout, int B, int M, int N, int K, int P, int TM, int TN, int TK, int TP>
+static int run_ke_fused(const void* a, const void* b, const void* c, void* d) {
+  using Traits = kernels::FusedTwoGemmsTraits<__half, float, WarpLayout, M, N, K, P, TM, TN, TK, TP>;
+  auto kern = k_ke_fused<Traits>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Traits::kSharedBytes) != hipSuccess) return -2;
+  hipLaunchKernelGGL(kern, dim3(M / TM, P / TP, B), dim3(Traits::kThreads), Traits::kSharedBytes, 0,
+                     static_cast<const __half*>(a), static_cast<const __half*>(b), static_cast<const __half*>(c),
+                     static_cast<__half*>(d));
+  return launch_status();
+}
+static const int kFusedShapes[4][5] = {{1, 256, 128, 64, 64}, {1, 1024, 256, 128, 128}, {3, 128, 64, 32, 32}, {2, 512, 128, 128, 256}};
+TT_API int tt_ke_fused(int variant, const void* a, const void* b, const void* c, void* d) {
+  switch (variant) {
+    case 0: return run_ke_fused<tl::RowMajor<2, 1>, 1, 256, 128, 64, 64, 64, 64, 64, 64>(a, b, c, d);
+    case 1: return run_ke_fused<tl::RowMajor<4, 1>, 1, 1024, 256, 128, 128, 64, 128, 128, 128>(a, b, c, d);
+    case 2: return run_ke_fused<tl::RowMajor<1, 1>, 3, 128, 64, 32, 32, 16, 32, 32, 16>(a, b, c, d);
+    case 3: return run_ke_fused<tl::RowMajor<4, 1>, 2, 512, 128, 128, 256, 128, 64, 32, 64>(a, b, c, d);
+    default: return -1;
+  }
+}
+TT_API void tt_ke_fused_shape(int variant, int* batch, int* m, int* n, int* k, int* p) {
+  const int* t = kFusedShapes[variant];
+  *batch = t[0]; *m = t[1]; *n = t[2]; *k = t[3]; *p = t[4];
+}
+
+// ---- 7. flash attention composed from the primitives (tests/python/test_flash_attn.py:
+//         (64,128,128,128) plain and (128,128,128,128) causal, tiles (64,128,128,128), 4 wavefronts) ---
+template <typename Traits>
+__global__ void k_ke_flash(const __half* q, const __half* k, const __half* v, __half* o) {
+  kernels::ke_flash_attention<__half, float, __half, Traits>(q, k, v, o);
+}
+template <typename WarpLayout, int B, int M, int N, int K, int P, int TM, int TN, int TK, int TP, bool kCausal>
+static int run_ke_flash(const void* q, const void* k, const void* v, void* o) {
+  // softmax scale 1/sqrt(K): K is 64 or 128 in every variant below
+  constexpr double kScale = K == 128 ? 0.08838834764831845 : 0.125;
+  using Traits = kernels::FlashAttentionTraits<__half, float, __half, TileShape<M, N, K, P>, TileShape<TM, TN, TK, TP>,
+                                               WarpLayout, kScale, kCausal>;
+  auto kern = k_ke_flash<Traits>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, Traits::kSharedBytes) != hipSuccess) return -2;
+  hipLaunchKernelGGL(kern, dim3(M / TM, P / TP, B), dim3(Traits::kThreads), Traits::kSharedBytes, 0,
+                     static_cast<const __half*>(q), static_cast<const __half*>(k), static_cast<const __half*>(v),
+                     static_cast<__half*>(o));
+  return launch_status();
+}
+static const int kFlashShapes[6][6] = {{1, 64, 128, 128, 128, 0},  {1, 128, 128, 128, 128, 1}, {2, 256, 512, 128, 128, 0},
+                                       {2, 512, 512, 64, 64, 1},   {1, 128, 256, 64, 128, 0},  {3, 256, 256, 128, 64, 1}};
+TT_API int tt_ke_flash(int variant, const void* q, const void* k, const void* v, void* o) {
+  switch (variant) {
+    case 0: return run_ke_flash<tl::RowMajor<4, 1>, 1, 64, 128, 128, 128, 64, 128, 128, 128, false>(q, k, v, o);
+    case 1: return run_ke_flash<tl::RowMajor<4, 1>, 1, 128, 128, 128, 128, 64, 128, 128, 128, true>(q, k, v, o);
+    case 2: return run_ke_flash<tl::RowMajor<4, 1>, 2, 256, 512, 128, 128, 64, 64, 128, 128, false>(q, k, v, o);
+    case 3: return run_ke_flash<tl::RowMajor<4, 1>, 2, 512, 512, 64, 64, 128, 64, 64, 64, true>(q, k, v, o);
+    case 4: return run_ke_flash<tl::RowMajor<2, 1>, 1, 128, 256, 64, 128, 32, 128, 32, 64, false>(q, k, v, o);
+    case 5: return run_ke_flash<tl::RowMajor<1, 1>, 3, 256, 256, 128, 64, 16, 32, 64, 32, true>(q, k, v, o);
+    default: return -1;
+  }
+}
+TT_API void tt_ke_flash_shape(int variant, int* batch, int* m, int* n, int* k, int* p, int* causal) {
+  const int* t = kFlashShapes[variant];
+  *batch = t[0]; *m = t[1]; *n = t[2]; *k = t[3]; *p = t[4]; *causal = t[5];
 }

@@ -1,5 +1,6 @@
 """GPU tests of the tile-programming headers (GlobalTile / SharedTile / RegTile, iterators,
-loaders / storers, gemm(), reduce / broadcast / map / mask, ke_gemm).  The kernels live in
+loaders / storers, gemm(), reduce / broadcast / map / mask, ke_gemm, ke_fused_two_gemms,
+ke_flash_attention).  The kernels live in
 tests/cpp/tile_api_kernels.hip and are driven through ctypes.
 
 Data-movement tests are bit-exact (integer-valued data `i % 2048` as in the reference's
@@ -38,6 +39,10 @@ def lib():
     lib.tt_ke_gemm.argtypes = [_i, _vp, _vp, _vp]
     lib.tt_ke_gemm_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 4
     lib.tt_softmax_pieces.argtypes = [_i, _vp, _vp, _vp, _vp, _i, _i]
+    lib.tt_ke_fused.argtypes = [_i, _vp, _vp, _vp, _vp]
+    lib.tt_ke_fused_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 5
+    lib.tt_ke_flash.argtypes = [_i, _vp, _vp, _vp, _vp]
+    lib.tt_ke_flash_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 6
     return lib
 
 
@@ -122,3 +127,38 @@ def test_reduce_broadcast_exp_mask(lib, variant, rows, cols, row_off, col_off):
     assert np.allclose(rsum.cpu().numpy()[keep], sm[keep], rtol=1e-5)
     want = 2 * e / np.where(keep, sm, 1)[:, None]
     assert np.allclose(out.cpu().numpy()[keep], want[keep], atol=1e-5)
+
+
+@pytest.mark.parametrize("variant", range(4))
+def test_ke_fused_two_gemms_composed_from_primitives(lib, variant):
+    # variant 0 is the reference's own case (tests/python/test_fused_two_gemms.py: 256,128,64,64)
+    bt, m, n, k, p = (_i(), _i(), _i(), _i(), _i())
+    lib.tt_ke_fused_shape(variant, bt, m, n, k, p)
+    g = torch.Generator().manual_seed(300 + variant)
+    a = (torch.randn(bt.value, m.value, k.value, generator=g) / 8).half()
+    b = (torch.randn(bt.value, n.value, k.value, generator=g) / 8).half()   # [n,k] buffer = col-major k x n
+    c = (torch.randn(bt.value, p.value, n.value, generator=g) / 8).half()   # [p,n] buffer = col-major n x p
+    d = torch.full((bt.value, m.value, p.value), float("nan"), dtype=torch.float16, device=DEV)
+    assert lib.tt_ke_fused(variant, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.to(DEV).data_ptr(), d.data_ptr()) == 0
+    for i in range(bt.value):
+        ref = N.fused_two_gemms_ref(a[i], b[i], c[i])
+        ok, r, ab = N.check_close(d[i], ref)
+        assert ok, (variant, i, r, ab)
+
+
+@pytest.mark.parametrize("variant", range(6))
+def test_ke_flash_attention_composed_from_primitives(lib, variant):
+    # variants 0 and 1 are the reference's own cases (tests/python/test_flash_attn.py:
+    # (64,128,128,128) plain, (128,128,128,128) causal; tiles (64,128,128,128))
+    bt, m, n, k, p, causal = (_i(), _i(), _i(), _i(), _i(), _i())
+    lib.tt_ke_flash_shape(variant, bt, m, n, k, p, causal)
+    g = torch.Generator().manual_seed(400 + variant)
+    q = torch.randn(bt.value, m.value, k.value, generator=g).half()
+    kk = torch.randn(bt.value, n.value, k.value, generator=g).half()
+    v = torch.randn(bt.value, n.value, p.value, generator=g).half()
+    vt = v.transpose(1, 2).contiguous()   # the kernel takes V column-major: a [p, n] buffer
+    o = torch.full((bt.value, m.value, p.value), float("nan"), dtype=torch.float16, device=DEV)
+    assert lib.tt_ke_flash(variant, q.to(DEV).data_ptr(), kk.to(DEV).data_ptr(), vt.to(DEV).data_ptr(), o.data_ptr()) == 0
+    ref = N.attention_ref(q, kk, v, causal=bool(causal.value))
+    ok, r, ab = N.check_close(o, ref)
+    assert ok, (variant, r, ab)

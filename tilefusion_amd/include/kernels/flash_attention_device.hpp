@@ -1,0 +1,213 @@
+// Flash-attention forward composed from the tile primitives (counterpart of
+// include/kernels/flash_attention_device.cuh:16-312): O[M,P] = softmax(scale * Q[M,K] K[K,N]
+// (+ causal mask)) V[N,P]; Q, O row-major, K and V column-major (V is handed over transposed,
+// as a [P][N] buffer); one workgroup per [kTM, kTP] tile of O, wavefronts stacked along M.
+//
+// Differences from the reference: running max / sum are fp32 and start at -inf / 0 (the
+// reference keeps them in fp16 and starts the max at 0); the output stays un-normalised until
+// the end (one divide instead of one per key tile); the causal mask skips key tiles that lie
+// entirely above the diagonal.  exp(S - max) is rounded to fp16 and re-laid-out through an LDS
+// tile for the second MFMA.  (The library's tuned entry point tf_flash_attention_fwd_f16
+// computes the scores transposed instead and needs no re-layout.)
+#pragma once
+
+#include "cell/mod.hpp"
+#include "types/mod.hpp"
+
+namespace tilefusion::kernels {
+using namespace tilefusion::cell;
+using namespace tilefusion::cell::copy;
+namespace tl = tile_layout;
+
+template <typename InType_, typename AccType_, typename OutType_, typename WholeShape, typename CtaTileShape,
+          typename WarpLayout_, double kSoftmaxScale_, bool kIsCausal_>
+struct FlashAttentionTraits {
+  using InType = InType_;
+  using AccType = AccType_;
+  using OutType = OutType_;
+  using WarpLayout = WarpLayout_;
+  static constexpr int kWarpPerRow = tl::num_rows<WarpLayout>;
+  static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
+  static_assert(kWarpPerCol == 1, "wavefronts must be arranged as a column vector");
+  static constexpr int kThreads = tl::get_numel<WarpLayout> * WARP_SIZE;
+  static constexpr int kSharedAccess = 64;
+  using BaseShape = BaseTileShape<InType>;
+
+  static constexpr int kM = dim_size<0, WholeShape>;  // query length
+  static constexpr int kN = dim_size<1, WholeShape>;  // key / value length
+  static constexpr int kK = dim_size<2, WholeShape>;  // query / key hidden dim
+  static constexpr int kP = dim_size<3, WholeShape>;  // value hidden dim
+  static constexpr int kTM = dim_size<0, CtaTileShape>;
+  static constexpr int kTN = dim_size<1, CtaTileShape>;
+  static constexpr int kTK = dim_size<2, CtaTileShape>;
+  static constexpr int kTP = dim_size<3, CtaTileShape>;
+  static_assert(kTK % 32 == 0 && kTN % 32 == 0 && kTP % 16 == 0 && (kTM / kWarpPerRow) % 16 == 0,
+                "tile sizes must be whole MFMA base tiles");
+  static constexpr double kSoftmaxScale = kSoftmaxScale_;
+  static constexpr bool kIsCausal = kIsCausal_;
+  static constexpr int kRowsPerWarp = kTM / kWarpPerRow;
+
+  using GlobalQ = GlobalTile<InType, tl::RowMajor<kTM, kK>>;
+  using GIteratorQ = GTileIterator<GlobalQ, TileShape<kTM, kTK>>;
+  using SharedQ = SharedTile<InType, tl::RowMajor<kTM, kTK>, true, kSharedAccess>;
+  using RegQ = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kRowsPerWarp / 16, kTK / 32>>;
+  using SharedQLoader = GlobalToSharedLoader<SharedQ, WarpLayout>;
+  using RegQLoader = SharedToRegLoader<RegQ, WarpLayout, WarpReuse::kRowReuseCont>;
+
+  using GlobalK = GlobalTile<InType, tl::ColMajor<kK, kN>>;
+  using GIteratorK = GTileIterator<GlobalK, TileShape<kTK, kTN>>;
+  using SharedK = SharedTile<InType, tl::ColMajor<kTK, kTN>, true, kSharedAccess>;
+  using RegK = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kTN / 16>>;
+  using SharedKLoader = GlobalToSharedLoader<SharedK, WarpLayout>;
+  using RegKLoader = SharedToRegLoader<RegK, WarpLayout, WarpReuse::kColReuseCont>;
+
+  using GlobalV = GlobalTile<InType, tl::ColMajor<kN, kTP>>;
+  using GIteratorV = GTileIterator<GlobalV, TileShape<kTN, kTP>>;
+  using SharedV = SharedTile<InType, tl::ColMajor<kTN, kTP>, true, kSharedAccess>;
+  using RegV = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTN / 32, kTP / 16>>;
+  using SharedVLoader = GlobalToSharedLoader<SharedV, WarpLayout>;
+  using RegVLoader = SharedToRegLoader<RegV, WarpLayout, WarpReuse::kColReuseCont>;
+
+  using GlobalO = GlobalTile<OutType, tl::RowMajor<kTM, kTP, kP>>;
+  using RegO = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kRowsPerWarp / 16, kTP / 16>>;
+  using RegOCast = RegTile<BaseTileAccRowMajor<OutType>, tl::RowMajor<kRowsPerWarp / 16, kTP / 16>>;
+  using ConvertO = compute::RegTileConvert<RegO, RegOCast>;
+  using OStorer = RegToGlobalStorer<GlobalO, RegOCast, WarpLayout>;
+
+  using RegAcc = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kRowsPerWarp / 16, kTN / 16>>;
+  using RegAccCast = RegTile<BaseTileAccRowMajor<InType>, tl::RowMajor<kRowsPerWarp / 16, kTN / 16>>;
+  using ConvertAcc = compute::RegTileConvert<RegAcc, RegAccCast>;
+  using SharedP = SharedTile<InType, tl::RowMajor<kTM, kTN>, true, kSharedAccess>;
+  using RegP = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kRowsPerWarp / 16, kTN / 32>>;
+  using StorerP = RegToSharedStorer<RegAccCast, WarpLayout>;
+  using LoaderP = SharedToRegLoader<RegP, WarpLayout, WarpReuse::kRowReuseCont>;
+
+  // one statistic per row a lane owns: 4 per base-tile row (fp32)
+  using RegVec = RegTile<AccType, tl::RowMajor<kRowsPerWarp / 16, 4>>;
+  using RowMax = compute::MaxReduce<RegAcc, tl::Layout::kRowMajor>;
+  using RowSum = compute::SumReduce<RegAcc, tl::Layout::kRowMajor>;
+  using BroadcastSub = compute::BroadcastSub<RegVec, RegAcc, tl::Layout::kRowMajor>;
+  using BroadcastMul = compute::BroadcastMul<RegVec, RegO, tl::Layout::kRowMajor>;
+  using BroadcastDiv = compute::BroadcastDiv<RegVec, RegO, tl::Layout::kRowMajor>;
+  using BlockExp = compute::RegTileExp<RegAcc>;
+  using VecMax = compute::BaseTileMax<RegVec>;
+  using VecAdd = compute::BaseTileAdd<RegVec>;
+  using VecSub = compute::BaseTileSub<RegVec>;
+  using VecMul = compute::BaseTileMul<RegVec>;
+  using VecExp = compute::BaseTileExp<RegVec>;
+  using ApplyMask = cell::ApplyMask<RegAcc, WarpLayout, BaseShape, MaskMode::kCausal>;
+  using ApplyScoreScale = compute::BroadcastScalarMul<RegAcc>;
+
+  static constexpr int kSharedBytes =
+      (SharedQ::kNumel + SharedK::kNumel + SharedV::kNumel + SharedP::kNumel) * (int)sizeof(InType);
+};
+
+template <typename InType, typename AccType, typename OutType, typename KeTraits>
+DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType* dV, OutType* dO) {
+  using T = KeTraits;
+  constexpr int kM = T::kM, kN = T::kN, kK = T::kK, kP = T::kP;
+  constexpr int kTM = T::kTM, kTN = T::kTN, kTP = T::kTP;
+  const InType* Q = dQ + ptrdiff_t(blockIdx.z) * kM * kK + ptrdiff_t(blockIdx.x) * kTM * kK;
+  const InType* K = dK + ptrdiff_t(blockIdx.z) * kK * kN;
+  const InType* V = dV + ptrdiff_t(blockIdx.z) * kN * kP + ptrdiff_t(blockIdx.y) * kTP * kN;
+  OutType* O = dO + ptrdiff_t(blockIdx.z) * kM * kP + ptrdiff_t(blockIdx.x) * kTM * kP + blockIdx.y * kTP;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char tilefusion_lds[];
+  InType* lds = reinterpret_cast<InType*>(tilefusion_lds);
+  typename T::SharedQ sQ(lds);
+  typename T::SharedK sK(lds + T::SharedQ::kNumel);
+  typename T::SharedV sV(lds + T::SharedQ::kNumel + T::SharedK::kNumel);
+  typename T::SharedP sP(lds + T::SharedQ::kNumel + T::SharedK::kNumel + T::SharedV::kNumel);
+
+  typename T::GIteratorQ gQs(Q);
+  typename T::GIteratorK gKs(K);
+  typename T::GIteratorV gVs(V);
+  typename T::SharedQLoader load_sq;
+  typename T::SharedKLoader load_sk;
+  typename T::SharedVLoader load_sv;
+  typename T::RegQLoader load_rq;
+  typename T::RegKLoader load_rk;
+  typename T::RegVLoader load_rv;
+  typename T::RegQ rQ;
+  typename T::RegK rK;
+  typename T::RegV rV;
+  typename T::RegP rP;
+  typename T::RegAcc s;
+  typename T::RegAccCast p_half;
+  typename T::RegO o;
+  typename T::RegVec run_max, run_sum, cur_max, cur_sum, new_max, alpha;
+#pragma unroll
+  for (int i = 0; i < T::RegVec::kNumel; ++i) run_max.mutable_data()[i] = -INFINITY;
+
+  const int row_base = blockIdx.x * kTM;
+  // causal: key tiles that start after the last row of this workgroup contribute nothing
+  const int n_tiles = T::kIsCausal ? min((int)T::GIteratorV::sc0, (row_base + kTM + kTN - 1) / kTN)
+                                   : (int)T::GIteratorV::sc0;
+  for (int n = 0; n < n_tiles; ++n) {
+    load_sv(gVs(n), sV);
+    for (int k = 0; k < T::GIteratorQ::sc1; ++k) {
+      load_sq(gQs(k), sQ);
+      load_sk(gKs(k, n), sK);
+      __copy_async();
+      __syncthreads();
+      load_rq(sQ, rQ);
+      load_rk(sK, rK);
+      compute::gemm(rQ, rK, s);
+      __syncthreads();
+    }
+    typename T::ApplyScoreScale scale;
+    scale(s, AccType(T::kSoftmaxScale), s);
+    if constexpr (T::kIsCausal) {
+      typename T::ApplyMask mask;
+      mask(s, row_base, n * kTN, -INFINITY);
+    }
+    typename T::RowMax row_max;
+    row_max(s, cur_max);
+    typename T::VecMax vmax;
+    vmax(cur_max, run_max, new_max);
+    // a row that is still fully masked keeps max = -inf; shift by 0 there so exp() sees -inf, not nan
+#pragma unroll
+    for (int i = 0; i < T::RegVec::kNumel; ++i) {
+      const AccType m = new_max.data()[i];
+      const AccType safe = (m == -INFINITY) ? AccType(0) : m;
+      alpha.mutable_data()[i] = __expf(run_max.data()[i] - safe);
+      cur_max.mutable_data()[i] = safe;
+    }
+    typename T::BroadcastSub sub;
+    sub(cur_max, s);
+    typename T::BlockExp block_exp;
+    block_exp(s, s);
+    typename T::RowSum row_sum;
+    row_sum(s, cur_sum);
+    typename T::VecMul vmul;
+    vmul(run_sum, alpha, run_sum);
+    typename T::VecAdd vadd;
+    vadd(run_sum, cur_sum, run_sum);
+    typename T::BroadcastMul rescale;
+    rescale(alpha, o);
+    copy_tile(new_max, run_max);
+
+    typename T::ConvertAcc to_half;
+    to_half(s, p_half);
+    typename T::StorerP store_p;
+    store_p(p_half, sP);
+    __copy_async();
+    __syncthreads();
+    typename T::LoaderP load_p;
+    load_p(sP, rP);
+    load_rv(sV, rV);
+    compute::gemm(rP, rV, o);
+    s.clear();
+    __syncthreads();
+  }
+  typename T::BroadcastDiv normalise;
+  normalise(run_sum, o);
+  typename T::RegOCast out;
+  typename T::ConvertO to_out;
+  to_out(o, out);
+  typename T::GlobalO gO(O);
+  typename T::OStorer store_o;
+  store_o(out, gO);
+}
+
+}  // namespace tilefusion::kernels
