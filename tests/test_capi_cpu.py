@@ -106,3 +106,13 @@ def test_op_schemas_match_the_reference():
     for name, schema in want.items():
         op = getattr(torch.ops.tilefusion, name).default
         assert str(op._schema) == schema
+
+
+def test_reference_package_name_imports_the_same_modules():
+    # callers written against the reference do `import tilefusion` / `from tilefusion.ops import gemm`
+    import tilefusion
+    import tilefusion_amd
+    from tilefusion.ops import flash_attention, fused_two_gemms, gemm
+    assert tilefusion.ops is tilefusion_amd.ops
+    assert gemm is tilefusion_amd.ops.gemm and fused_two_gemms is tilefusion_amd.ops.fused_two_gemms
+    assert flash_attention is tilefusion_amd.ops.flash_attention

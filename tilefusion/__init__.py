@@ -1,0 +1,13 @@
+"""`import tilefusion` for callers written against the reference package name
+(python/__init__.py:19-40): the same modules as `tilefusion_amd`, under the reference's name."""
+
+import sys
+
+import tilefusion_amd
+from tilefusion_amd import __version__, ops  # noqa: F401
+
+sys.modules[__name__ + ".ops"] = ops
+for _name in ("gemm", "fused_two_gemms", "flash_attention", "flash_decode"):
+    sys.modules[f"{__name__}.ops.{_name}"] = sys.modules[f"tilefusion_amd.ops.{_name}"]
+
+__all__ = ["ops"]

@@ -9,6 +9,7 @@
 // (__copy_async() + __syncthreads()), like with the reference's cp.async version.
 #pragma once
 
+#include "cell/copy/copy_atom.hpp"
 #include "cell/copy/warp.hpp"
 #include "types/global.hpp"
 #include "types/shared.hpp"
@@ -54,8 +55,8 @@ struct GlobalToSharedLoader {
     for (int v = threadIdx.x; v < Walk::kVectors; v += Walk::kThreads) {
       int r, c;
       Walk::coord(v, r, c);
-      const uint4 val = *reinterpret_cast<const uint4*>(g + ptrdiff_t(r) * Global::kRowStride + ptrdiff_t(c) * Global::kColStride);
-      *reinterpret_cast<uint4*>(s + dst.fetch_physical_offset(r * Shared::kRowStride + c * Shared::kColStride)) = val;
+      atom::ld_global_st_shared<16>(s + dst.fetch_physical_offset(r * Shared::kRowStride + c * Shared::kColStride),
+                                    g + ptrdiff_t(r) * Global::kRowStride + ptrdiff_t(c) * Global::kColStride);
     }
   }
 };
@@ -77,8 +78,8 @@ struct SharedToGlobalStorer {
     for (int v = threadIdx.x; v < Walk::kVectors; v += Walk::kThreads) {
       int r, c;
       Walk::coord(v, r, c);
-      const uint4 val = *reinterpret_cast<const uint4*>(s + src.fetch_physical_offset(r * Shared::kRowStride + c * Shared::kColStride));
-      *reinterpret_cast<uint4*>(g + ptrdiff_t(r) * Global::kRowStride + ptrdiff_t(c) * Global::kColStride) = val;
+      atom::ld_shared_st_global<16>(g + ptrdiff_t(r) * Global::kRowStride + ptrdiff_t(c) * Global::kColStride,
+                                    s + src.fetch_physical_offset(r * Shared::kRowStride + c * Shared::kColStride));
     }
   }
 };

@@ -1,6 +1,7 @@
 #pragma once
 
 #include "cell/copy/constants.hpp"
+#include "cell/copy/copy_atom.hpp"
 #include "cell/copy/global_to_register.hpp"
 #include "cell/copy/global_to_shared.hpp"
 #include "cell/copy/register.hpp"
