@@ -32,14 +32,16 @@ PEAK_FP16_TFLOPS = 2516.6   # 256 CU x 2.4 GHz x 4096 flop/clk/CU (dense fp16 MF
 PEAK_HBM_GBS = 8000.0       # HBM3E, 8 TB/s
 
 
-PRE_WARM_MS = 150.0  # the GPU takes ~100 ms of sustained load to settle its clocks
+PRE_WARM_MS = 300.0
 
 
-def _time_steps(fn, steps, warmup):
+def _time_steps(fn, steps, warmup, pre_warm_ms=PRE_WARM_MS):
     import torch
-    # Untimed pre-warm so that the W warm-up steps start from settled clocks: short benchmarks
-    # otherwise time the power-management ramp (first ~100 ms are 10-20% slower).
-    t_end = time.perf_counter() + PRE_WARM_MS / 1e3
+    # Untimed pre-warm with the kernel under test so that the W warm-up steps start from the
+    # clocks this kernel settles at: the power management needs a few hundred ms of sustained
+    # load to converge (launch durations first swing by 10-20%), and a different pre-warm load
+    # would leave the clocks where THAT load settles.
+    t_end = time.perf_counter() + pre_warm_ms / 1e3
     i = 0
     while time.perf_counter() < t_end:
         fn(i)
@@ -271,12 +273,38 @@ def _capi():
     return m
 
 
-def run_workload(w, steps, warmup, with_cpu):
+class Copy:
+    """Calibration only: a plain device-to-device copy of known size, the yardstick the
+    FETCH_SIZE / WRITE_SIZE counters of the other workloads are scaled by."""
+    name = "copy_1gib"
+    metric, unit, bound = "copy_gbs", "GB/s", "hbm"
+    nbytes = 1 << 30
+    bytes = 2 * nbytes
+    flops = 0.0
+    traffic = None
+    config = {"workload": "torch copy_ of 1 GiB (reads 1 GiB, writes 1 GiB)", "inputs": "uint8 zeros"}
+
+    def setup(self, dev):
+        import torch
+        self.src = torch.zeros(self.nbytes, device=dev, dtype=torch.uint8)
+        self.dst = torch.empty_like(self.src)
+
+    def step(self, i):
+        self.dst.copy_(self.src)
+
+    def check(self):
+        return True, 0.0, 0.0
+
+    def cpu_baseline(self):
+        return {"value": 0.0, "unit": "GB/s", "sample": "none"}
+
+
+def run_workload(w, steps, warmup, with_cpu, pre_warm_ms=PRE_WARM_MS):
     import torch
     dev = "cuda:0"
     w.setup(dev)
     ok, rel, mabs = w.check()
-    ms, wall_ms = _time_steps(w.step, steps, warmup)
+    ms, wall_ms = _time_steps(w.step, steps, warmup, pre_warm_ms)
     if w.bound == "mfma":
         achieved, peak, runit = w.flops / ms / 1e9, PEAK_FP16_TFLOPS, "TFLOP/s"
     else:
@@ -285,7 +313,7 @@ def run_workload(w, steps, warmup, with_cpu):
         "metric": w.metric, "value": round(achieved, 2), "unit": w.unit, "ms_per_step": round(ms, 5),
         "wall_ms_per_step": round(wall_ms, 5),
         "roofline": {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": runit,
-                     "frac": round(achieved / peak, 4), "traffic": None},
+                     "frac": round(achieved / peak, 4), "traffic": getattr(w, "traffic", None)},
         "tflops": round(w.flops / ms / 1e9, 2), "algorithmic_gbs": round(w.bytes / ms / 1e6, 1),
         "parity": {"ok": bool(ok), "rel_l2": float("%.3e" % rel), "max_abs": float("%.3e" % mabs),
                    "tolerance": "rel_l2<=1e-3, max_abs<=2e-2 vs fp32 CPU oracle"},
@@ -308,12 +336,14 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "gemm", "fused", "attention", "attention_causal", "decode"])
+                    choices=["all", "gemm", "fused", "attention", "attention_causal", "decode", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--prewarm-ms", type=float, default=PRE_WARM_MS,
+                    help="untimed run of the kernel under test before each workload (0 for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the hot path on ONE GPU; --gpus N with N > 1 is not supported "
-              "(see DESIGN.md for how each kernel would shard).", file=sys.stderr)
+              "(every kernel shards over independent rows / heads without exchange).", file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():
@@ -321,9 +351,9 @@ def main():
         sys.exit(1)
     torch.set_num_threads(max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))))
     table = {"gemm": Gemm4096(), "fused": Fused(), "attention": Attention(False),
-             "attention_causal": Attention(True), "decode": Decode()}
+             "attention_causal": Attention(True), "decode": Decode(), "copy": Copy()}
     head_key = "gemm" if args.workload == "all" else args.workload
-    head = run_workload(table[head_key], args.steps, args.warmup, not args.no_cpu)
+    head = run_workload(table[head_key], args.steps, args.warmup, not args.no_cpu and head_key != "copy", args.prewarm_ms)
     prop = torch.cuda.get_device_properties(0)
     line = {
         "metric": head["metric"], "value": head["value"], "unit": head["unit"], "n_gpus": 1,
@@ -339,7 +369,7 @@ def main():
         others = {}
         for key in ("fused", "attention", "attention_causal", "decode"):
             steps = args.steps if key != "decode" else max(5, min(args.steps, 20))
-            others[key] = run_workload(table[key], steps, min(args.warmup, 5), not args.no_cpu)
+            others[key] = run_workload(table[key], steps, min(args.warmup, 5), not args.no_cpu, args.prewarm_ms)
         line["workloads"] = others
     print(json.dumps(line))
 

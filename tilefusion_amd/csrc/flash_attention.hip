@@ -68,7 +68,7 @@ TFK_DEVICE half4_t lds_read_tr4(const char* p) {
 template <int D, int DV, bool kVT, bool kCausal, int kWavesT>
 __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-    half_t* __restrict__ O, int Lq, int Lkv, float scale_log2, int q_tiles) {
+    half_t* __restrict__ O, int Lq, int Lkv, float scale_log2, int q_tiles, int total_items) {
   constexpr int kBMq = kWavesT * 32;
   constexpr int kKChunks = D / 8;
   constexpr int kVChunks = kVT ? kBN / 8 : DV / 8;
@@ -87,11 +87,35 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 31, lg = lane >> 5;
-  // Non-causal: x = query tile, y = slice.  Causal: x = slice, y = query tile with the heaviest
-  // (latest) tiles dispatched first across ALL slices, so the tail of the grid is made of the
-  // cheapest workgroups.
-  const int qt = kCausal ? (q_tiles - 1 - (int)blockIdx.y) : (int)blockIdx.x;
-  const size_t bh = kCausal ? blockIdx.x : blockIdx.y;
+  // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: id % 8 is the XCD,
+  // id / 8 the position in that XCD's queue.  Work is arranged so that the query tiles of a
+  // slice stream the same K/V through ONE L2 instead of eight.
+  //   non-causal: items in slice-major order, cut into 8 contiguous chunks (the last one may
+  //               be short; its surplus workgroups exit at once);
+  //   causal:     work per query tile varies 1..q_tiles, so every queue is sorted
+  //               heaviest (latest) tile first across the slices it owns; with a slice count
+  //               that is not a multiple of 8 the queues would be unequal, so the order falls
+  //               back to heaviest-first over all slices.
+  int qt;
+  size_t bh;
+  if (!kCausal) {
+    const int per_xcd = (total_items + 7) / 8;
+    const int item = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+    if (item >= total_items) return;
+    qt = item % q_tiles;
+    bh = item / q_tiles;
+  } else {
+    if ((int)blockIdx.x >= total_items) return;
+    const int slices = total_items / q_tiles;
+    if (slices % 8 == 0) {
+      const int per = slices / 8, slot = blockIdx.x / 8;
+      qt = q_tiles - 1 - slot / per;
+      bh = (blockIdx.x % 8) * per + slot % per;
+    } else {
+      qt = q_tiles - 1 - (int)blockIdx.x / slices;
+      bh = blockIdx.x % slices;
+    }
+  }
   Q += bh * (size_t)Lq * D;
   K += bh * (size_t)Lkv * D;
   V += bh * (size_t)Lkv * DV;
@@ -342,11 +366,12 @@ int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, in
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
   constexpr int bm = kWavesT * 32;
   const int q_tiles = (Lq + bm - 1) / bm;
-  const dim3 grid = kCausal ? dim3(batch, q_tiles) : dim3(q_tiles, batch);
+  const int total_items = q_tiles * batch;
+  const dim3 grid(8 * ((total_items + 7) / 8));
   hipLaunchKernelGGL(kern, grid, dim3(kWavesT * 64), lds, st,
                      static_cast<const half_t*>(Q), static_cast<const half_t*>(K),
                      static_cast<const half_t*>(V), static_cast<half_t*>(O), Lq, Lkv, scale_log2,
-                     q_tiles);
+                     q_tiles, total_items);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
 }
