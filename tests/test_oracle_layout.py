@@ -172,3 +172,23 @@ def test_mfma_fragment_maps_cover_tiles():
                               (L.mfma_16x16x32_ab, L.mfma_16x16x32_c, 16, 32, 4)]:
         assert {ab(l, t) for l in range(64) for t in range(8)} == {(i, kk) for i in range(m) for kk in range(k)}
         assert {c(l, r) for l in range(64) for r in range(nreg)} == {(i, j) for i in range(m) for j in range(m)}
+
+
+def test_golden_fixture():
+    # tests/golden/layout_known_answers.json: the reference's asserted integers, as data
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "layout_known_answers.json")) as f:
+        g = json.load(f)
+    mk = {"RowMajor": L.row_major, "ColMajor": L.col_major}
+    for m in g["matrix_layouts"]:
+        lay = mk[m["kind"]](m["rows"], m["cols"])
+        assert (lay.numel, lay.row_stride, lay.col_stride, lay.kind) == (m["numel"], m["row_stride"], m["col_stride"], m["kind"])
+    for b in g["block_layouts"]:
+        lay = L.BlockMatrixLayout(mk[b["outer"][0]](*b["outer"][1:]), mk[b["inner"][0]](*b["inner"][1:]))
+        assert (lay.tile_rows, lay.tile_cols, lay.row_stride, lay.col_stride, lay.kind) == (
+            b["tile_rows"], b["tile_cols"], b["row_stride"], b["col_stride"], b["kind"])
+        for i, j, off in b["samples"]:
+            assert lay(i, j) == off
+    for x, y, want in g["swizzle_3_3_3_points"]:
+        assert L.swizzle(x * 64 + y, 3, 3, 3) == want
