@@ -56,10 +56,26 @@ TFK_DEVICE float pair_sum(float x) {
 
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 
-TFK_DEVICE half4_t lds_read_tr4(const char* p) {
+// `addr` is a 32-bit LDS byte address: integer arithmetic on it (base register + constant)
+// folds into the instruction's offset field, pointer arithmetic through a generic pointer
+// does not.
+TFK_DEVICE half4_t lds_read_tr4(unsigned addr) {
   fp16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
-      (__attribute__((address_space(3))) fp16x4_t*)(p));
+      (__attribute__((address_space(3))) fp16x4_t*)(size_t)addr);
   return __builtin_bit_cast(half4_t, v);
+}
+TFK_DEVICE half4_t lds_read_b64(unsigned addr) {
+  return *(__attribute__((address_space(3))) const half4_t*)(size_t)addr;
+}
+TFK_DEVICE half8_t lds_read_b128(unsigned addr) {
+  return *(__attribute__((address_space(3))) const half8_t*)(size_t)addr;
+}
+// Hides how `x` was computed from the optimiser.  Without it the loop-invariant part of
+// (stage base + lane offset + constant) is hoisted as one register per read and the constant
+// never reaches the offset field.
+TFK_DEVICE unsigned opaque(unsigned x) {
+  asm volatile("" : "+v"(x));
+  return x;
 }
 
 // kWavesT wavefronts x 32 queries per workgroup.  8 wavefronts (256 queries) halve the
@@ -220,7 +236,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   };
   auto process_tile = [&](int it, auto mask_c) __attribute__((always_inline)) {
     constexpr bool kMask = decltype(mask_c)::value;
-    const unsigned stage_off = (it % kStages) * kStageBytes;
+    const unsigned stage_base = smem_base + (it % kStages) * kStageBytes;
     const int n0 = it * kBN;
     // ---- S^T = K Q^T ------------------------------------------------------------------
     float16_t s[kNT];
@@ -230,10 +246,10 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       for (int r = 0; r < 16; ++r) s[nt][r] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < D / 16; ++kk) {
-      const char* kb = smem + (stage_off + k_off[kk]);
+      const unsigned kb = opaque(stage_base + k_off[kk]);
 #pragma unroll
       for (int nt = 0; nt < kNT; ++nt) {
-        const half8_t kf = *reinterpret_cast<const half8_t*>(kb + nt * 32 * D * 2);
+        const half8_t kf = lds_read_b128(kb + nt * 32 * D * 2);
         s[nt] = mfma_32x32x16(kf, qf[kk], s[nt]);
       }
     }
@@ -274,20 +290,19 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       m_run = m_new;
     }
     const float mc = m_run * c;
-    float psum = 0.f;
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        s[nt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][r], c, -mc));
-        psum += s[nt][r];
-      }
-    l_run += psum;
+      for (int r = 0; r < 16; ++r) s[nt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][r], c, -mc));
 
     // ---- O^T += V^T P^T ---------------------------------------------------------------
-    const char* vb[kVOffs];
+    // The row sum is taken over the fp16-rounded weights, the values that actually multiply
+    // V (v_dot2_f32_f16 against (1, 1): two weights per instruction, fp32 accumulate).
+    unsigned vb[kVOffs];
 #pragma unroll
-    for (int x = 0; x < kVOffs; ++x) vb[x] = smem + (stage_off + kKBytes + v_off[x]);
+    for (int x = 0; x < kVOffs; ++x) vb[x] = opaque(stage_base + v_off[x]) + kKBytes;
+    const half2_t ones = {(half_t)1.f, (half_t)1.f};
+    float psum = 0.f;
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
@@ -297,6 +312,10 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
         half8_t pb;
 #pragma unroll
         for (int t = 0; t < 8; ++t) pb[t] = (half_t)s[nt][8 * j + t];
+        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 0, 1), ones, psum, false);
+        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 2, 3), ones, psum, false);
+        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 4, 5), ones, psum, false);
+        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 6, 7), ones, psum, false);
         const int nk = nt * 32 + 16 * j;
 #pragma unroll
         for (int dt = 0; dt < kDT; ++dt) {
@@ -305,8 +324,8 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
             lo = lds_read_tr4(vb[dt] + nk * DV * 2);
             hi = lds_read_tr4(vb[dt] + (nk + 8) * DV * 2);
           } else {
-            lo = *reinterpret_cast<const half4_t*>(vb[nk / 8] + dt * 32 * kBN * 2);
-            hi = *reinterpret_cast<const half4_t*>(vb[nk / 8 + 1] + dt * 32 * kBN * 2);
+            lo = lds_read_b64(vb[nk / 8] + dt * 32 * kBN * 2);
+            hi = lds_read_b64(vb[nk / 8 + 1] + dt * 32 * kBN * 2);
           }
           half8_t vf;
 #pragma unroll
@@ -317,6 +336,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
           o_acc[dt] = mfma_32x32x16(vf, pb, o_acc[dt]);
         }
       }
+    l_run += psum;
   };
 
   // Tiles [0, n_plain) need no mask for this wavefront's 32 rows, [n_plain, n_compute) cross
