@@ -5,12 +5,15 @@
 // include/cell/mask.hpp:75-82) and its host launcher (src/kernels/flash_attn.cu:58-152).
 // CDNA4 design (FA-2 style, un-normalised O with one divide at the end):
 //   * one workgroup = 256 queries (8 wavefronts x 32; 4 x 32 for short query ranges),
-//     key/value tiles of 64 rows, v_mfma_f32_32x32x16_f16 throughout;
+//     key/value tiles of 64 rows, v_mfma_f32_16x16x32_f16 throughout (the most
+//     power-efficient fp16 MFMA shape: the kernel runs at the power limit, so energy per
+//     flop sets its speed);
 //   * Q stays in registers for the whole workgroup (the reference reloads it per KV tile);
-//   * scores are computed transposed, S^T = K Q^T, so a lane owns ONE query row: its 32
-//     score values per tile are plain registers, the row max / sum is an in-lane reduction
-//     plus a single v_permlane32_swap with the partner lane, and exp2(S^T) converted to fp16
-//     is already the B-operand fragment of the second MFMA O^T = V^T P^T;
+//   * scores are computed transposed, S^T = K Q^T, so a lane owns one query row per 16-query
+//     block: its score values are plain registers, the running max / sum are in-lane
+//     reductions (the 4 lanes that share a query only talk when the reference max moves),
+//     and exp2(S^T) converted to fp16 is already the B-operand fragment of the second MFMA
+//     O^T = V^T P^T;
 //   * K and V tiles go global -> LDS directly (global_load_lds_dwordx4) into a 3-stage ring;
 //     V is kept [key][dim] in LDS and transposed on the way to registers with
 //     ds_read_b64_tr_b16; both tiles are XOR-swizzled against bank conflicts;
@@ -25,33 +28,19 @@ namespace {
 constexpr int kBN = 64;   // keys per tile
 constexpr int kStages = 3;
 
-// K tile [kBN][D]: 16 consecutive rows reading one logical chunk hit 16 bank groups.
+// K tile [kBN][D] (and a transposed V tile [DV][kBN]): 16 consecutive rows reading one logical
+// 16-byte chunk hit 16 different bank groups.
 template <int CH>
 __host__ __device__ constexpr int swz_k(int row, int c) {
   constexpr int kRowsPer256B = CH >= 16 ? 1 : 16 / CH;
   return c ^ ((row / kRowsPer256B) % CH);
 }
-// V tile [kBN][DV] read by transposing 4-row x 16-column blocks: 4 consecutive rows must land
-// in different 64-byte quarters of the bank space.
+// V tile [kBN][DV] read by transposing 4-row x 16-column blocks: a half wavefront touches 8
+// rows x 32 bytes at the same column, which must land in 8 different 32-byte bank windows.
 template <int CH>
 __host__ __device__ constexpr int swz_v(int row, int c) {
-  if constexpr (CH >= 16) return c ^ ((row & 3) << 2);
-  return c ^ (((row >> 1) & 1) << 2);
-}
-
-// v_permlane32_swap hands every lane its own value and the value of lane l ^ 32 (in an order
-// that depends on the half the lane sits in), which is all a symmetric reduction needs.
-TFK_DEVICE float pair_max(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x),
-                                            __builtin_bit_cast(unsigned, x), false, false);
-  const unsigned a = r[0], b = r[1];  // copy out: bit_cast of a vector element is unreliable
-  return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
-}
-TFK_DEVICE float pair_sum(float x) {
-  auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, x),
-                                            __builtin_bit_cast(unsigned, x), false, false);
-  const unsigned a = r[0], b = r[1];
-  return __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b);
+  if constexpr (CH >= 16) return c ^ ((row & 7) << 1);
+  return c ^ (((row >> 1) & 3) << 1);
 }
 
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
@@ -77,6 +66,15 @@ TFK_DEVICE unsigned opaque(unsigned x) {
   asm volatile("" : "+v"(x));
   return x;
 }
+// Reductions over the 4 lanes l, l^16, l^32, l^48 that share a query (rare path / epilogue).
+TFK_DEVICE float quad_max(float x) {
+  x = fmaxf(x, __shfl_xor(x, 16));
+  return fmaxf(x, __shfl_xor(x, 32));
+}
+TFK_DEVICE float quad_sum(float x) {
+  x += __shfl_xor(x, 16);
+  return x + __shfl_xor(x, 32);
+}
 
 // kWavesT wavefronts x 32 queries per workgroup.  8 wavefronts (256 queries) halve the
 // K/V traffic per query and put two wavefronts on every SIMD, so one wavefront's softmax
@@ -91,8 +89,11 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   constexpr int kKBytes = kBN * D * 2;
   constexpr int kVBytes = kBN * DV * 2;
   constexpr int kStageBytes = kKBytes + kVBytes;
-  constexpr int kNT = kBN / 32;
-  constexpr int kDT = DV / 32;
+  constexpr int kQB = 2;          // 16-query blocks per wavefront
+  constexpr int kKB = kBN / 16;   // 16-key blocks per tile (rows of S^T)
+  constexpr int kKK = D / 32;     // reduction steps of S^T = K Q^T
+  constexpr int kDB = DV / 16;    // 16-wide blocks of the head dimension (rows of O^T)
+  constexpr int kJ = kBN / 32;    // reduction steps of O^T += V^T P^T
   constexpr int kKInstr = kKBytes / 1024;            // 1 KiB wavefront loads per K tile
   constexpr int kVInstr = kVBytes / 1024;
   constexpr int kKPerWave = (kKInstr + kWavesT - 1) / kWavesT;
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int lr = lane & 31, lg = lane >> 5;
+  const int lr = lane & 15, lg = lane >> 4;
   // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2: id % 8 is the XCD,
   // id / 8 the position in that XCD's queue.  Work is arranged so that the query tiles of a
   // slice stream the same K/V through ONE L2 instead of eight.
@@ -138,17 +139,21 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   O += bh * (size_t)Lq * DV;
 
   const int q_row0 = qt * kBMq + wave * 32;  // first query row of this wavefront
-  const int m_row = q_row0 + lr;             // this lane's query row
-  const int m_ld = min(m_row, Lq - 1);
+  // this lane's query rows: block qb holds row q_row0 + 16*qb + lr
 
   // A negative scale is folded into Q (scores change sign, the scale becomes positive), so
   // that the running maximum can be taken on raw scores and scaled once per row.
   const float c = fmaxf(fabsf(scale_log2), 1e-30f);  // (a zero scale still yields uniform weights)
-  half8_t qf[D / 16];
+  // Q^T fragments (B operand): lane holds Q[row][32*kk + 8*lg .. +7]
+  half8_t qf[kKK][kQB];
 #pragma unroll
-  for (int kk = 0; kk < D / 16; ++kk) {
-    qf[kk] = *reinterpret_cast<const half8_t*>(Q + (size_t)m_ld * D + kk * 16 + lg * 8);
-    if (scale_log2 < 0.f) qf[kk] = -qf[kk];
+  for (int qb = 0; qb < kQB; ++qb) {
+    const int m_ld = min(q_row0 + 16 * qb + lr, Lq - 1);
+#pragma unroll
+    for (int kk = 0; kk < kKK; ++kk) {
+      qf[kk][qb] = *reinterpret_cast<const half8_t*>(Q + (size_t)m_ld * D + kk * 32 + lg * 8);
+      if (scale_log2 < 0.f) qf[kk][qb] = -qf[kk][qb];
+    }
   }
 
   int n_end = Lkv;
@@ -191,37 +196,47 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   // Every fragment read is (stage base) + (per-lane offset) + (compile-time immediate): the
   // swizzles only XOR lane-dependent bits into the chunk index, so the lane part is computed
   // once here and the tile loop spends no VALU on addresses beyond adding the stage base.
-  //   K fragment (nt, kk): row 32*nt + lr, logical chunk 2*kk + lg.
-  unsigned k_off[D / 16];
+  //   K fragment (kb, kk) - A operand, 16 keys x 32 dims: row 16*kb + lr, logical chunk 4*kk + lg.
+  unsigned k_off[kKK];
 #pragma unroll
-  for (int kk = 0; kk < D / 16; ++kk) k_off[kk] = lr * D * 2 + swz_k<kKChunks>(lr, 2 * kk + lg) * 16;
-  //   V fragment (dt, keys nk..nk+15), V kept [key][dim]: a 16-lane group transposes the 4 x 16
-  //   block of rows nk + 4*lg (+8) .. +3, columns 32*dt + 16*((lane>>4)&1) .. +15; lane r of the
-  //   group addresses row r/4, columns 4*(r%4) .. +3 of that block.
-  //   V^T fragment, V kept [dim][key]: row 32*dt + lr, keys nk + 4*lg (+8) .. +3.
-  constexpr int kVOffs = kVT ? 8 : kDT;
+  for (int kk = 0; kk < kKK; ++kk) k_off[kk] = lr * D * 2 + swz_k<kKChunks>(lr, 4 * kk + lg) * 16;
+  //   Reduction step j of the second product covers keys 32*j .. +31; slot t of lane group lg
+  //   is key 32*j + 4*lg + t (t < 4) or 32*j + 16 + 4*lg + (t - 4): exactly the keys whose
+  //   scores the lane already holds in its accumulators of key blocks 2*j and 2*j + 1.
+  //   V fragment (db, j) - A operand, 16 dims x 32 keys.
+  //     V kept [key][dim]: each 16-lane group transposes the 4 x 16 block of rows
+  //     32*j + 4*lg (+16) .. +3, columns 16*db .. +15; lane r of the group addresses row r/4,
+  //     columns 4*(r%4) .. +3 of that block.  One offset per (db & 1, db / 2 via XOR) would not
+  //     be constant, so the lane part is kept per db.
+  //     V kept [dim][key]: row 16*db + lr, keys 32*j + 4*lg (+16) .. +3 (8 bytes each).
+  constexpr int kVOffs = kVT ? 2 * kJ : kDB;
   unsigned v_off[kVOffs];
   if constexpr (!kVT) {
-    const int r16 = lane & 15;
-    const int row_l = 4 * lg + (r16 >> 2);
-    const int col_l = 16 * ((lane >> 4) & 1) + 4 * (r16 & 3);
+    const int row_l = 4 * lg + (lr >> 2);
 #pragma unroll
-    for (int dt = 0; dt < kDT; ++dt) {
-      const int col = dt * 32 + col_l;
-      v_off[dt] = row_l * DV * 2 + swz_v<kVChunks>(row_l, col / 8) * 16 + (col % 8) * 2;
+    for (int db = 0; db < kDB; ++db) {
+      const int col = db * 16 + 4 * (lr & 3);
+      v_off[db] = row_l * DV * 2 + swz_v<kVChunks>(row_l, col / 8) * 16 + (col % 8) * 2;
     }
   } else {
 #pragma unroll
-    for (int cc = 0; cc < 8; ++cc) v_off[cc] = lr * kBN * 2 + swz_k<kVChunks>(lr, cc) * 16 + lg * 8;
+    for (int x = 0; x < 2 * kJ; ++x) {  // x = 2*j + half: keys 32*j + 16*half + 4*lg .. +3
+      const int key = 16 * x + 4 * lg;
+      v_off[x] = lr * kBN * 2 + swz_k<kVChunks>(lr, key / 8) * 16 + (key % 8) * 2;
+    }
   }
 
-  float16_t o_acc[kDT];
+  float4_t o_acc[kDB][kQB];
 #pragma unroll
-  for (int dt = 0; dt < kDT; ++dt)
+  for (int db = 0; db < kDB; ++db)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o_acc[dt][r] = 0.f;
-  float m_run = -INFINITY;  // reference max of the raw (sign-adjusted) scores (see below)
-  float l_run = 0.f;        // this lane's share of the running sum
+    for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run[kQB], l_run[kQB];  // reference max of the raw scores; this lane's share of the sum
+#pragma unroll
+  for (int qb = 0; qb < kQB; ++qb) {
+    m_run[qb] = -INFINITY;
+    l_run[qb] = 0.f;
+  }
 
   // Ring of kStages tiles: tile it+kStages-1 is requested at the top of iteration it.
 #pragma unroll
@@ -238,62 +253,74 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     constexpr bool kMask = decltype(mask_c)::value;
     const unsigned stage_base = smem_base + (it % kStages) * kStageBytes;
     const int n0 = it * kBN;
-    // ---- S^T = K Q^T ------------------------------------------------------------------
-    float16_t s[kNT];
+    // ---- S^T = K Q^T: s[kb][qb][r] = score(key n0 + 16*kb + 4*lg + r, query block qb row lr) --
+    float4_t s[kKB][kQB];
 #pragma unroll
-    for (int nt = 0; nt < kNT; ++nt)
+    for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[nt][r] = 0.f;
+      for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int kk = 0; kk < D / 16; ++kk) {
-      const unsigned kb = opaque(stage_base + k_off[kk]);
+    for (int kk = 0; kk < kKK; ++kk) {
+      const unsigned ka = opaque(stage_base + k_off[kk]);
 #pragma unroll
-      for (int nt = 0; nt < kNT; ++nt) {
-        const half8_t kf = lds_read_b128(kb + nt * 32 * D * 2);
-        s[nt] = mfma_32x32x16(kf, qf[kk], s[nt]);
+      for (int kb = 0; kb < kKB; ++kb) {
+        const half8_t kf = lds_read_b128(ka + kb * 16 * D * 2);
+#pragma unroll
+        for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = mfma_16x16x32(kf, qf[kk][qb], s[kb][qb]);
       }
     }
 
     // ---- mask -------------------------------------------------------------------------
-    // s[nt][r] is the score of key n0 + 32*nt + 8*(r/4) + 4*lg + r%4 against query m_row
     if constexpr (kMask) {
 #pragma unroll
-      for (int nt = 0; nt < kNT; ++nt)
+      for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int n = n0 + nt * 32 + 8 * (r / 4) + 4 * lg + (r % 4);
-          if (n >= Lkv || (kCausal && n > m_row)) s[nt][r] = -INFINITY;
-        }
+        for (int qb = 0; qb < kQB; ++qb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int n = n0 + kb * 16 + 4 * lg + r;
+            if (n >= Lkv || (kCausal && n > q_row0 + 16 * qb + lr)) s[kb][qb][r] = -INFINITY;
+          }
     }
 
     // ---- online softmax: p = exp2(c*s - c*m) -------------------------------------------
-    float mx = s[0][0];
-#pragma unroll
-    for (int nt = 0; nt < kNT; ++nt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nt][r]);
-    mx = pair_max(mx);
-    // Lazy rescale: exponents are taken against a reference m_run that is only raised when a
-    // row's maximum has grown by more than kLazy (in log2 units) since the reference was set.
-    // Until then p = 2^(c*(s - m_run)) may reach 2^kLazy, which fp16 P and the fp32 sums hold
-    // easily, and the final O / l is unchanged because O and l share the reference.  Raising
-    // it costs a multiply of every O accumulator, so this skips it on almost every tile.
+    // Lazy reference: exponents are taken against m_run, which is only raised when some
+    // lane's maximum has grown by more than kLazy (in log2 units) past it.  Until then
+    // p = 2^(c*(s - m_run)) may reach 2^kLazy, which fp16 P and the fp32 sums hold easily, and
+    // the final O / l is unchanged because O and l share the reference.  The check needs no
+    // cross-lane traffic: it looks at each lane's own 16 keys; only when it fires are the 4
+    // lanes that share a query reduced and every O accumulator multiplied.
     constexpr float kLazy = 8.f;
-    if (__builtin_amdgcn_ballot_w64((mx - m_run) * c > kLazy) != 0) {
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
-      l_run *= alpha;
+    float mx[kQB];
+    bool grow = false;
 #pragma unroll
-      for (int dt = 0; dt < kDT; ++dt)
+    for (int qb = 0; qb < kQB; ++qb) {
+      mx[qb] = s[0][qb][0];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o_acc[dt][r] *= alpha;
-      m_run = m_new;
+      for (int kb = 0; kb < kKB; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mx[qb] = fmaxf(mx[qb], s[kb][qb][r]);
+      grow |= (mx[qb] - m_run[qb]) * c > kLazy;
     }
-    const float mc = m_run * c;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
-    for (int nt = 0; nt < kNT; ++nt)
+      for (int qb = 0; qb < kQB; ++qb) {
+        const float m_new = fmaxf(m_run[qb], quad_max(mx[qb]));
+        const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c);
+        l_run[qb] *= alpha;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s[nt][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[nt][r], c, -mc));
+        for (int db = 0; db < kDB; ++db) o_acc[db][qb] *= alpha;
+        m_run[qb] = m_new;
+      }
+    }
+#pragma unroll
+    for (int qb = 0; qb < kQB; ++qb) {
+      const float mc = m_run[qb] * c;
+#pragma unroll
+      for (int kb = 0; kb < kKB; ++kb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) s[kb][qb][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][r], c, -mc));
+    }
 
     // ---- O^T += V^T P^T ---------------------------------------------------------------
     // The row sum is taken over the fp16-rounded weights, the values that actually multiply
@@ -302,41 +329,43 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
     for (int x = 0; x < kVOffs; ++x) vb[x] = opaque(stage_base + v_off[x]) + kKBytes;
     const half2_t ones = {(half_t)1.f, (half_t)1.f};
-    float psum = 0.f;
 #pragma unroll
-    for (int nt = 0; nt < kNT; ++nt)
+    for (int j = 0; j < kJ; ++j) {
+      half8_t pb[kQB];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        // reduction step over keys nk .. nk+15; slot t of lane group lg is key
-        // nk + 4*lg + t (t < 4) or nk + 8 + 4*lg + (t - 4)
-        half8_t pb;
+      for (int qb = 0; qb < kQB; ++qb) {
 #pragma unroll
-        for (int t = 0; t < 8; ++t) pb[t] = (half_t)s[nt][8 * j + t];
-        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 0, 1), ones, psum, false);
-        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 2, 3), ones, psum, false);
-        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 4, 5), ones, psum, false);
-        psum = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb, pb, 6, 7), ones, psum, false);
-        const int nk = nt * 32 + 16 * j;
-#pragma unroll
-        for (int dt = 0; dt < kDT; ++dt) {
-          half4_t lo, hi;
-          if constexpr (!kVT) {
-            lo = lds_read_tr4(vb[dt] + nk * DV * 2);
-            hi = lds_read_tr4(vb[dt] + (nk + 8) * DV * 2);
-          } else {
-            lo = lds_read_b64(vb[nk / 8] + dt * 32 * kBN * 2);
-            hi = lds_read_b64(vb[nk / 8 + 1] + dt * 32 * kBN * 2);
-          }
-          half8_t vf;
-#pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            vf[t] = lo[t];
-            vf[4 + t] = hi[t];
-          }
-          o_acc[dt] = mfma_32x32x16(vf, pb, o_acc[dt]);
+        for (int t = 0; t < 4; ++t) {
+          pb[qb][t] = (half_t)s[2 * j][qb][t];
+          pb[qb][4 + t] = (half_t)s[2 * j + 1][qb][t];
         }
+        float ps = l_run[qb];
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 0, 1), ones, ps, false);
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 2, 3), ones, ps, false);
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 4, 5), ones, ps, false);
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 6, 7), ones, ps, false);
+        l_run[qb] = ps;
       }
-    l_run += psum;
+#pragma unroll
+      for (int db = 0; db < kDB; ++db) {
+        half4_t lo, hi;
+        if constexpr (!kVT) {
+          lo = lds_read_tr4(vb[db] + (32 * j) * DV * 2);
+          hi = lds_read_tr4(vb[db] + (32 * j + 16) * DV * 2);
+        } else {
+          lo = lds_read_b64(vb[2 * j] + db * 16 * kBN * 2);
+          hi = lds_read_b64(vb[2 * j + 1] + db * 16 * kBN * 2);
+        }
+        half8_t vf;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          vf[t] = lo[t];
+          vf[4 + t] = hi[t];
+        }
+#pragma unroll
+        for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = mfma_16x16x32(vf, pb[qb], o_acc[db][qb]);
+      }
+    }
   };
 
   // Tiles [0, n_plain) need no mask for this wavefront's 32 rows, [n_plain, n_compute) cross
@@ -360,19 +389,20 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   for (; it < num_tiles; ++it) ring_step(it);
   wait_vmem_all();  // the clamped tail loads must not outlive the workgroup's LDS
 
-  // ---- epilogue: O[m][d] = O^T[d][m] / l --------------------------------------------------
-  const float l_tot = pair_sum(l_run);
-  const float inv = 1.f / l_tot;
-  if (m_row < Lq) {
+  // ---- epilogue: O[m][16*db + 4*lg + r] = O^T / l ------------------------------------------
 #pragma unroll
-    for (int dt = 0; dt < kDT; ++dt)
+  for (int qb = 0; qb < kQB; ++qb) {
+    const float inv = 1.f / quad_sum(l_run[qb]);
+    const int m_row = q_row0 + 16 * qb + lr;
+    if (m_row < Lq) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int db = 0; db < kDB; ++db) {
         half4_t out;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) out[t] = (half_t)(o_acc[dt][4 * q + t] * inv);
-        *reinterpret_cast<half4_t*>(O + (size_t)m_row * DV + dt * 32 + 8 * q + 4 * lg) = out;
+        for (int t = 0; t < 4; ++t) out[t] = (half_t)(o_acc[db][qb][t] * inv);
+        *reinterpret_cast<half4_t*>(O + (size_t)m_row * DV + db * 16 + 4 * lg) = out;
       }
+    }
   }
 }
 
