@@ -141,18 +141,20 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   const int q_row0 = qt * kBMq + wave * 32;  // first query row of this wavefront
   // this lane's query rows: block qb holds row q_row0 + 16*qb + lr
 
-  // A negative scale is folded into Q (scores change sign, the scale becomes positive), so
-  // that the running maximum can be taken on raw scores and scaled once per row.
-  const float c = fmaxf(fabsf(scale_log2), 1e-30f);  // (a zero scale still yields uniform weights)
-  // Q^T fragments (B operand): lane holds Q[row][32*kk + 8*lg .. +7]
+  // The softmax scale (times log2 e) is folded into Q once: Q' = fp16(Q * scale_log2), so the
+  // MFMA result is already in log2 units; and each score accumulator starts at minus the
+  // row's reference maximum instead of zero, so the MFMA result IS the exp2 argument - no
+  // per-score multiply or subtract is left in the tile loop.
+  // Q^T fragments (B operand): lane holds Q'[row][32*kk + 8*lg .. +7]
   half8_t qf[kKK][kQB];
 #pragma unroll
   for (int qb = 0; qb < kQB; ++qb) {
     const int m_ld = min(q_row0 + 16 * qb + lr, Lq - 1);
 #pragma unroll
     for (int kk = 0; kk < kKK; ++kk) {
-      qf[kk][qb] = *reinterpret_cast<const half8_t*>(Q + (size_t)m_ld * D + kk * 32 + lg * 8);
-      if (scale_log2 < 0.f) qf[kk][qb] = -qf[kk][qb];
+      const half8_t raw = *reinterpret_cast<const half8_t*>(Q + (size_t)m_ld * D + kk * 32 + lg * 8);
+#pragma unroll
+      for (int t = 0; t < 8; ++t) qf[kk][qb][t] = (half_t)((float)raw[t] * scale_log2);
     }
   }
 
@@ -231,10 +233,12 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   for (int db = 0; db < kDB; ++db)
 #pragma unroll
     for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
-  float m_run[kQB], l_run[kQB];  // reference max of the raw scores; this lane's share of the sum
+  // neg_m: minus the reference maximum of a row's scaled scores (the accumulator start value);
+  // l_run: this lane's share of the running sum of weights.
+  float neg_m[kQB], l_run[kQB];
 #pragma unroll
   for (int qb = 0; qb < kQB; ++qb) {
-    m_run[qb] = -INFINITY;
+    neg_m[qb] = 0.f;  // reference 0 until the first tile raises it
     l_run[qb] = 0.f;
   }
 
@@ -253,12 +257,13 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     constexpr bool kMask = decltype(mask_c)::value;
     const unsigned stage_base = smem_base + (it % kStages) * kStageBytes;
     const int n0 = it * kBN;
-    // ---- S^T = K Q^T: s[kb][qb][r] = score(key n0 + 16*kb + 4*lg + r, query block qb row lr) --
+    // ---- S^T = K Q'^T - m: s[kb][qb][r] = log2-scaled score of key n0 + 16*kb + 4*lg + r
+    //      against row lr of query block qb, minus that row's reference maximum --------------
     float4_t s[kKB][kQB];
 #pragma unroll
     for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
-      for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
+      for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = float4_t{neg_m[qb], neg_m[qb], neg_m[qb], neg_m[qb]};
 #pragma unroll
     for (int kk = 0; kk < kKK; ++kk) {
       const unsigned ka = opaque(stage_base + k_off[kk]);
@@ -283,13 +288,13 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
           }
     }
 
-    // ---- online softmax: p = exp2(c*s - c*m) -------------------------------------------
-    // Lazy reference: exponents are taken against m_run, which is only raised when some
-    // lane's maximum has grown by more than kLazy (in log2 units) past it.  Until then
-    // p = 2^(c*(s - m_run)) may reach 2^kLazy, which fp16 P and the fp32 sums hold easily, and
-    // the final O / l is unchanged because O and l share the reference.  The check needs no
-    // cross-lane traffic: it looks at each lane's own 16 keys; only when it fires are the 4
-    // lanes that share a query reduced and every O accumulator multiplied.
+    // ---- online softmax: p = exp2(s) ---------------------------------------------------
+    // Lazy reference: the reference maximum is only raised when some lane sees a score more
+    // than kLazy (log2 units) above it.  Until then p may reach 2^kLazy, which fp16 P and the
+    // fp32 sums hold easily, and the final O / l is unchanged because O and l share the
+    // reference.  The check needs no cross-lane traffic: it looks at each lane's own 16 keys;
+    // only when it fires are the 4 lanes that share a query reduced, every O accumulator
+    // multiplied and this tile's scores re-based.
     constexpr float kLazy = 8.f;
     float mx[kQB];
     bool grow = false;
@@ -300,27 +305,31 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) mx[qb] = fmaxf(mx[qb], s[kb][qb][r]);
-      grow |= (mx[qb] - m_run[qb]) * c > kLazy;
+      grow |= mx[qb] > kLazy;
     }
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+    // The first tile sets the reference to the row's true maximum, whichever way that is from
+    // the initial 0 (every row has at least key 0 unmasked there; nothing is accumulated yet).
+    const bool first = it == 0;
+    if (first || __builtin_amdgcn_ballot_w64(grow) != 0) {
 #pragma unroll
       for (int qb = 0; qb < kQB; ++qb) {
-        const float m_new = fmaxf(m_run[qb], quad_max(mx[qb]));
-        const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c);
+        const float qmax = quad_max(mx[qb]);
+        const float shift = first ? qmax : fmaxf(0.f, qmax);  // afterwards the reference only rises
+        const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-shift);
         l_run[qb] *= alpha;
 #pragma unroll
         for (int db = 0; db < kDB; ++db) o_acc[db][qb] *= alpha;
-        m_run[qb] = m_new;
+#pragma unroll
+        for (int kb = 0; kb < kKB; ++kb) s[kb][qb] -= shift;
+        neg_m[qb] -= shift;
       }
     }
 #pragma unroll
-    for (int qb = 0; qb < kQB; ++qb) {
-      const float mc = m_run[qb] * c;
+    for (int qb = 0; qb < kQB; ++qb)
 #pragma unroll
       for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) s[kb][qb][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][qb][r], c, -mc));
-    }
+        for (int r = 0; r < 4; ++r) s[kb][qb][r] = __builtin_amdgcn_exp2f(s[kb][qb][r]);
 
     // ---- O^T += V^T P^T ---------------------------------------------------------------
     // The row sum is taken over the fp16-rounded weights, the values that actually multiply
