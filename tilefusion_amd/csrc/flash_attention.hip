@@ -14,7 +14,7 @@
 //     reductions (the 4 lanes that share a query only talk when the reference max moves),
 //     and exp2(S^T) converted to fp16 is already the B-operand fragment of the second MFMA
 //     O^T = V^T P^T;
-//   * K and V tiles go global -> LDS directly (global_load_lds_dwordx4) into a 3-stage ring;
+//   * K and V tiles go global -> LDS directly (global_load_lds_dwordx4) into a 4-stage ring;
 //     V is kept [key][dim] in LDS and transposed on the way to registers with
 //     ds_read_b64_tr_b16; both tiles are XOR-swizzled against bank conflicts;
 //   * causal: tiles right of the diagonal are skipped, only tiles crossing it are masked.
@@ -26,7 +26,7 @@ namespace tfk {
 namespace {
 
 constexpr int kBN = 64;   // keys per tile
-constexpr int kStages = 3;
+constexpr int kStages = 4;
 
 // K tile [kBN][D] (and a transposed V tile [DV][kBN]): 16 consecutive rows reading one logical
 // 16-byte chunk hit 16 different bank groups.
@@ -79,17 +79,17 @@ TFK_DEVICE float quad_sum(float x) {
 // kWavesT wavefronts x 32 queries per workgroup.  8 wavefronts (256 queries) halve the
 // K/V traffic per query and put two wavefronts on every SIMD, so one wavefront's softmax
 // (VALU) overlaps the other's MFMAs; 4 wavefronts serve short query ranges.
-template <int D, int DV, bool kVT, bool kCausal, int kWavesT>
+template <int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQB>
 __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
     half_t* __restrict__ O, int Lq, int Lkv, float scale_log2, int q_tiles, int total_items) {
-  constexpr int kBMq = kWavesT * 32;
+  constexpr int kRowsPerWave = 16 * kQB;  // kQB 16-query blocks per wavefront
+  constexpr int kBMq = kWavesT * kRowsPerWave;
   constexpr int kKChunks = D / 8;
   constexpr int kVChunks = kVT ? kBN / 8 : DV / 8;
   constexpr int kKBytes = kBN * D * 2;
   constexpr int kVBytes = kBN * DV * 2;
   constexpr int kStageBytes = kKBytes + kVBytes;
-  constexpr int kQB = 2;          // 16-query blocks per wavefront
   constexpr int kKB = kBN / 16;   // 16-key blocks per tile (rows of S^T)
   constexpr int kKK = D / 32;     // reduction steps of S^T = K Q^T
   constexpr int kDB = DV / 16;    // 16-wide blocks of the head dimension (rows of O^T)
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   V += bh * (size_t)Lkv * DV;
   O += bh * (size_t)Lq * DV;
 
-  const int q_row0 = qt * kBMq + wave * 32;  // first query row of this wavefront
+  const int q_row0 = qt * kBMq + wave * kRowsPerWave;  // first query row of this wavefront
   // this lane's query rows: block qb holds row q_row0 + 16*qb + lr
 
   // The softmax scale (times log2 e) is folded into Q once: Q' = fp16(Q * scale_log2), so the
@@ -242,39 +242,73 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     l_run[qb] = 0.f;
   }
 
-  // Ring of kStages tiles: tile it+kStages-1 is requested at the top of iteration it.
+  // Ring of kStages tiles.  Iteration `it` starts with the ring step: wait until tile it+1 has
+  // landed (only the loads of younger tiles stay in flight), meet the other wavefronts, then
+  // request tile it+kStages-1 into the stage of tile it-1, which nobody reads any more.  Tile
+  // it+1 is needed that early because the wavefronts of a workgroup run in two phases (below).
 #pragma unroll
   for (int t = 0; t < kStages - 1; ++t) issue_tile_loads(t);
-
-  // Every iteration starts with the ring step: tile `it` has landed once only the younger
-  // tiles' loads are outstanding; the barrier also tells us every wavefront is done with
-  // tile it-1, whose stage is re-filled next.
+  barrier_keep_vmem<(kStages - 2) * kLoadsPerTile>();  // tile 0 has landed
   auto ring_step = [&](int it) __attribute__((always_inline)) {
-    barrier_keep_vmem<(kStages - 2) * kLoadsPerTile>();
+    barrier_keep_vmem<(kStages - 3) * kLoadsPerTile>();
     issue_tile_loads(it + kStages - 1);
   };
-  auto process_tile = [&](int it, auto mask_c) __attribute__((always_inline)) {
-    constexpr bool kMask = decltype(mask_c)::value;
+  float4_t s[kKB][kQB];  // scores of the tile in flight (carried across iterations by late wavefronts)
+  // Operand fragments are requested from LDS one step ahead of the MFMAs that use them, into
+  // ping-pong registers, so that LDS latency is covered by the previous step's MFMAs (or by
+  // the softmax arithmetic) instead of stalling the wavefront in front of every MFMA group.
+  half8_t kf[2][kKB];   // K fragments of reduction step kk (buffer kk & 1)
+  half8_t vf[2][kDB];   // V fragments of reduction step j (buffer j & 1)
+  auto k_reads = [&](int buf, int it, int kk) __attribute__((always_inline)) {
+    const unsigned ka = opaque(smem_base + (it % kStages) * kStageBytes + k_off[kk]);
+#pragma unroll
+    for (int kb = 0; kb < kKB; ++kb) kf[buf][kb] = lds_read_b128(ka + kb * 16 * D * 2);
+  };
+  auto v_reads = [&](int buf, int it, int j) __attribute__((always_inline)) {
     const unsigned stage_base = smem_base + (it % kStages) * kStageBytes;
-    const int n0 = it * kBN;
-    // ---- S^T = K Q'^T - m: s[kb][qb][r] = log2-scaled score of key n0 + 16*kb + 4*lg + r
-    //      against row lr of query block qb, minus that row's reference maximum --------------
-    float4_t s[kKB][kQB];
+#pragma unroll
+    for (int db = 0; db < kDB; ++db) {
+      half4_t lo, hi;
+      if constexpr (!kVT) {
+        const unsigned va = opaque(stage_base + v_off[db]) + kKBytes;
+        lo = lds_read_tr4(va + (32 * j) * DV * 2);
+        hi = lds_read_tr4(va + (32 * j + 16) * DV * 2);
+      } else {
+        lo = lds_read_b64(opaque(stage_base + v_off[2 * j]) + kKBytes + db * 16 * kBN * 2);
+        hi = lds_read_b64(opaque(stage_base + v_off[2 * j + 1]) + kKBytes + db * 16 * kBN * 2);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        vf[buf][db][t] = lo[t];
+        vf[buf][db][4 + t] = hi[t];
+      }
+    }
+  };
+  // ---- S^T = K Q'^T - m: s[kb][qb][r] = log2-scaled score of key 64*it + 16*kb + 4*lg + r
+  //      against row lr of query block qb, minus that row's reference maximum.  Expects the
+  //      fragments of step kk = 0 to be on their way into kf[0]. ---------------------------
+  auto qk_tile = [&](int it) __attribute__((always_inline)) {
 #pragma unroll
     for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
       for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = float4_t{neg_m[qb], neg_m[qb], neg_m[qb], neg_m[qb]};
 #pragma unroll
     for (int kk = 0; kk < kKK; ++kk) {
-      const unsigned ka = opaque(stage_base + k_off[kk]);
+      if (kk + 1 < kKK) k_reads((kk + 1) & 1, it, kk + 1);
 #pragma unroll
-      for (int kb = 0; kb < kKB; ++kb) {
-        const half8_t kf = lds_read_b128(ka + kb * 16 * D * 2);
+      for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
-        for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = mfma_16x16x32(kf, qf[kk][qb], s[kb][qb]);
-      }
+        for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = mfma_16x16x32(kf[kk & 1][kb], qf[kk][qb], s[kb][qb]);
+      __builtin_amdgcn_sched_barrier(0);
     }
-
+  };
+  half8_t pb[kJ][kQB];  // fp16 weights, B operand of the second product
+  // ---- mask, online softmax, fp16 weights.  Requests the V fragments of step j = 0. -------
+  auto softmax_tile = [&](int it, auto mask_c) __attribute__((always_inline)) {
+    constexpr bool kMask = decltype(mask_c)::value;
+    const int n0 = it * kBN;
+    v_reads(0, it, 0);
+    __builtin_amdgcn_sched_barrier(0);
     // ---- mask -------------------------------------------------------------------------
     if constexpr (kMask) {
 #pragma unroll
@@ -331,69 +365,86 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) s[kb][qb][r] = __builtin_amdgcn_exp2f(s[kb][qb][r]);
 
-    // ---- O^T += V^T P^T ---------------------------------------------------------------
     // The row sum is taken over the fp16-rounded weights, the values that actually multiply
     // V (v_dot2_f32_f16 against (1, 1): two weights per instruction, fp32 accumulate).
-    unsigned vb[kVOffs];
-#pragma unroll
-    for (int x = 0; x < kVOffs; ++x) vb[x] = opaque(stage_base + v_off[x]) + kKBytes;
     const half2_t ones = {(half_t)1.f, (half_t)1.f};
 #pragma unroll
-    for (int j = 0; j < kJ; ++j) {
-      half8_t pb[kQB];
+    for (int j = 0; j < kJ; ++j)
 #pragma unroll
       for (int qb = 0; qb < kQB; ++qb) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          pb[qb][t] = (half_t)s[2 * j][qb][t];
-          pb[qb][4 + t] = (half_t)s[2 * j + 1][qb][t];
+          pb[j][qb][t] = (half_t)s[2 * j][qb][t];
+          pb[j][qb][4 + t] = (half_t)s[2 * j + 1][qb][t];
         }
         float ps = l_run[qb];
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 0, 1), ones, ps, false);
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 2, 3), ones, ps, false);
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 4, 5), ones, ps, false);
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[qb], pb[qb], 6, 7), ones, ps, false);
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 0, 1), ones, ps, false);
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 2, 3), ones, ps, false);
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 4, 5), ones, ps, false);
+        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 6, 7), ones, ps, false);
         l_run[qb] = ps;
       }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // ---- O^T += V^T P^T; during its last step the K fragments (kk = 0) of tile `it_next`
+  //      are requested for the QK phase that follows ------------------------------------------
+  auto pv_tile = [&](int it, int it_next) __attribute__((always_inline)) {
 #pragma unroll
-      for (int db = 0; db < kDB; ++db) {
-        half4_t lo, hi;
-        if constexpr (!kVT) {
-          lo = lds_read_tr4(vb[db] + (32 * j) * DV * 2);
-          hi = lds_read_tr4(vb[db] + (32 * j + 16) * DV * 2);
-        } else {
-          lo = lds_read_b64(vb[2 * j] + db * 16 * kBN * 2);
-          hi = lds_read_b64(vb[2 * j + 1] + db * 16 * kBN * 2);
-        }
-        half8_t vf;
+    for (int j = 0; j < kJ; ++j) {
+      if (j + 1 < kJ) v_reads((j + 1) & 1, it, j + 1);
+      else k_reads(0, it_next, 0);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          vf[t] = lo[t];
-          vf[4 + t] = hi[t];
-        }
+      for (int db = 0; db < kDB; ++db)
 #pragma unroll
-        for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = mfma_16x16x32(vf, pb[qb], o_acc[db][qb]);
-      }
+        for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = mfma_16x16x32(vf[j & 1][db], pb[j][qb], o_acc[db][qb]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Tiles [0, n_plain) need no mask for this wavefront's 32 rows, [n_plain, n_compute) cross
+  // Tiles [0, n_plain) need no mask for this wavefront's rows, [n_plain, n_compute) cross
   // the diagonal or the end of the keys, and [n_compute, num_tiles) lie above the diagonal:
   // the wavefront only keeps the ring (barrier + loads) going for its workgroup.
   int n_plain = min(num_tiles, Lkv / kBN);
   int n_compute = num_tiles;
   if (kCausal) {
     n_plain = max(0, min(n_plain, (q_row0 + 1) / kBN));
-    n_compute = min(num_tiles, (q_row0 + 31) / kBN + 1);
+    n_compute = min(num_tiles, (q_row0 + kRowsPerWave - 1) / kBN + 1);
   }
+  // Two wavefronts share a SIMD (w and w + 4).  If both ran QK -> softmax -> PV in lockstep
+  // (the per-tile barrier aligns them), they would fight for the MFMA pipe in two phases and
+  // leave it idle while both do their softmax.  So the second wavefront of each SIMD runs one
+  // phase late - softmax(it), PV(it), QK(it+1) between the same barriers - and its softmax
+  // overlaps the first one's QK MFMAs, the first one's softmax its PV MFMAs.
+  const bool late = kWavesT == 8 && wave >= 4;
   int it = 0;
-  for (; it < n_plain; ++it) {
-    ring_step(it);
-    process_tile(it, std::false_type{});
-  }
-  for (; it < n_compute; ++it) {
-    ring_step(it);
-    process_tile(it, std::true_type{});
+  k_reads(0, 0, 0);
+  if (!late) {
+    for (; it < n_plain; ++it) {
+      ring_step(it);
+      qk_tile(it);
+      softmax_tile(it, std::false_type{});
+      pv_tile(it, it + 1);
+    }
+    for (; it < n_compute; ++it) {
+      ring_step(it);
+      qk_tile(it);
+      softmax_tile(it, std::true_type{});
+      pv_tile(it, it + 1);
+    }
+  } else {
+    qk_tile(0);
+    for (; it < n_plain; ++it) {
+      ring_step(it);
+      softmax_tile(it, std::false_type{});
+      pv_tile(it, it + 1);
+      if (it + 1 < n_compute) qk_tile(it + 1);
+    }
+    for (; it < n_compute; ++it) {
+      ring_step(it);
+      softmax_tile(it, std::true_type{});
+      pv_tile(it, it + 1);
+      if (it + 1 < n_compute) qk_tile(it + 1);
+    }
   }
   for (; it < num_tiles; ++it) ring_step(it);
   wait_vmem_all();  // the clamped tail loads must not outlive the workgroup's LDS
@@ -415,15 +466,15 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   }
 }
 
-template <int D, int DV, bool kVT, bool kCausal, int kWavesT>
+template <int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQB>
 int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
              float scale_log2, hipStream_t st) {
-  auto kern = flash_attention_fwd_kernel<D, DV, kVT, kCausal, kWavesT>;
+  auto kern = flash_attention_fwd_kernel<D, DV, kVT, kCausal, kWavesT, kQB>;
   constexpr int lds = kStages * (kBN * D * 2 + kBN * DV * 2);
   static_assert(lds <= kMaxLdsBytes, "tiles do not fit in LDS");
   TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-  constexpr int bm = kWavesT * 32;
+  constexpr int bm = kWavesT * 16 * kQB;
   const int q_tiles = (Lq + bm - 1) / bm;
   const int total_items = q_tiles * batch;
   const dim3 grid(8 * ((total_items + 7) / 8));
@@ -438,8 +489,11 @@ int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, in
 template <int D, int DV, bool kVT, bool kCausal>
 int launch(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
            float scale_log2, hipStream_t st) {
-  if (Lq > 128) return launch_w<D, DV, kVT, kCausal, 8>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
-  return launch_w<D, DV, kVT, kCausal, 4>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+#ifndef TFK_FA_BIG
+#define TFK_FA_BIG 8, 2
+#endif
+  if (Lq > 128) return launch_w<D, DV, kVT, kCausal, TFK_FA_BIG>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+  return launch_w<D, DV, kVT, kCausal, 4, 2>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
 }
 
 template <int D, int DV>
