@@ -59,6 +59,28 @@ def test_scale_and_large_logits():
         assert ok, f"scale={scale}: rel_l2={r:.3e} max_abs={m:.3e}"
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_reference_maximum_moves_both_ways(causal):
+    # The kernel starts every score at minus a lazily updated reference maximum.  Keys whose
+    # scores are far below zero first, far above later (and the reverse) force the reference
+    # down on the first tile and up by hundreds of log2 units afterwards; a stale reference
+    # would underflow every weight to 0 (division by zero) or overflow fp16.
+    g = torch.Generator().manual_seed(99)
+    d, lq, lkv = 128, 256, 512
+    q = torch.randn(1, lq, d, generator=g).half()
+    k = torch.randn(1, lkv, d, generator=g).half()
+    v = torch.randn(1, lkv, d, generator=g).half()
+    q[..., 0] = 8.0                       # a strong common component ...
+    ramp = torch.linspace(-6.0, 6.0, lkv)  # ... that the keys weight from very negative to very positive
+    for direction in (1.0, -1.0):
+        k2 = k.clone()
+        k2[0, :, 0] = (direction * ramp).half()
+        o = c_attention(q.to(DEV), k2.to(DEV), v.to(DEV), causal, 1.0)   # scale 1: logits span +-48
+        assert not torch.isnan(o).any() and not torch.isinf(o).any()
+        ok, r, m = N.check_close(o, N.attention_ref(q, k2, v, scale=1.0, causal=causal))
+        assert ok, f"direction={direction}: rel_l2={r:.3e} max_abs={m:.3e}"
+
+
 def test_invariants():
     q, k, v = _inputs(2, 256, 256, 128, 5)
     # causal row 0 sees only key 0
