@@ -83,6 +83,29 @@ TF_API int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void
                                int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
                                void* stream);
 
+/* Run-time compilation of kernels written against the tile headers (tilefusion_amd/include),
+ * for shapes that are template parameters there.  tf_jit_compile builds `source` with
+ * `hipcc --genco` for gfx950 (the tile headers are on the include path; include_paths and
+ * compile_args are appended to the defaults), caches the code object on disk by content hash
+ * and in the process by (hash, kernel_name), and returns the handle of the `extern "C"
+ * __global__` function `kernel_name`.  tf_jit_launch enqueues it: kernel_args is the usual
+ * array of pointers to the argument values.  A failed compile returns TF_ERR_HIP and leaves
+ * the compiler's output in tf_last_error().
+ * Replaces: tilefusion::jit::JitCompiler::compile_kernel / get_or_compile_kernel
+ * (include/jit/compiler.hpp:21-81, src/jit/compiler.cc:123-225) and the cuLaunchKernel calls
+ * of the host launchers (src/kernels/gemm.cu:136-141). */
+TF_API int tf_jit_compile(const char* kernel_name, const char* source,
+                          const char* const* include_paths, int num_include_paths,
+                          const char* const* compile_args, int num_compile_args,
+                          void** kernel_out);
+TF_API int tf_jit_launch(void* kernel, unsigned grid_x, unsigned grid_y, unsigned grid_z,
+                         unsigned block_x, unsigned block_y, unsigned block_z,
+                         unsigned dynamic_lds_bytes, void* stream, void** kernel_args);
+/* Drops the in-process kernel cache (JitCompiler::clear_cache, src/jit/compiler.cc:147-163). */
+TF_API int tf_jit_clear_cache(void);
+/* Directory of the on-disk code-object cache. */
+TF_API const char* tf_jit_cache_dir(void);
+
 /* Message of the last failing call on this thread ("" if none). */
 TF_API const char* tf_last_error(void);
 /* Library version string, e.g. "tilefusion-mi355x 0.1.0 (gfx950)". */

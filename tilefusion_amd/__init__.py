@@ -33,6 +33,6 @@ def _load_library(filename: str) -> Any:
 
 _lib = _load_library("libtilefusion.so")
 
-from . import _capi, ops  # noqa: E402
+from . import _capi, jit, ops  # noqa: E402
 
-__all__ = ["ops"]
+__all__ = ["jit", "ops"]

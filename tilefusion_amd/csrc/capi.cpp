@@ -5,7 +5,7 @@
 
 namespace tfk {
 namespace {
-thread_local char g_last_error[512] = "";
+thread_local char g_last_error[4096] = "";  // room for a compiler diagnostic
 }
 
 void set_error(const char* fmt, ...) {
