@@ -83,6 +83,18 @@ TF_API int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void
                                int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
                                void* stream);
 
+/* data[indices[i, 0..index_depth-1], ...] += updates[i, ...] for every index row i; duplicate
+ * rows accumulate (atomic adds), rows that point outside `data` are skipped.  `data` has
+ * `rank` dimensions data_dims (host array, row-major, contiguous); indices is a device
+ * [num_index_rows, index_depth] int64 array; updates is [num_index_rows, prod(data_dims[
+ * index_depth..])].  dtype: 0 fp32, 1 fp16, 2 bf16.  Nothing is allocated (the reference
+ * cudaMallocs the strides on every call and leaks them).
+ * Replaces: tilefusion::kernels::scatter_nd, src/kernels/scatter_nd.cu:36-95
+ * (schema include/kernels/kernel_list.hpp:11-13). */
+TF_API int tf_scatter_nd(const void* updates, void* data, const int64_t* indices,
+                         const int64_t* data_dims, int rank, int64_t num_index_rows,
+                         int index_depth, int dtype, void* stream);
+
 /* Run-time compilation of kernels written against the tile headers (tilefusion_amd/include),
  * for shapes that are template parameters there.  tf_jit_compile builds `source` with
  * `hipcc --genco` for gfx950 (the tile headers are on the include path; include_paths and

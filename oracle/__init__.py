@@ -20,6 +20,8 @@ sign/index or transposed operand):
 * flash_decode_ref / split_kv_partials / combine_partials - q_len = 1 closed form; the
   split + log-sum-exp combine identity is pinned against the direct form for random split
   counts.  These have NO counterpart in the reference (it has no decoding kernel).
+* scatter_nd_ref - torch index_put_(accumulate=True) (library routine), pinned against a
+  hand-written loop on a tiny case in tests/test_oracle_numerics.py.
 * layout oracles (oracle/layout.py) - pinned by the reference's integer known answers
   (tests/cpp/types/test_layout.cu, test_swizzle.cu, test_gtile_iterator.cu,
   test_warp_base_tile_shape.cu), restated in tests/test_oracle_layout.py.
@@ -38,6 +40,7 @@ from .numerics import (  # noqa: F401
     fused_two_gemms_ref,
     fused_two_gemms_ref_rounded,
     attention_ref,
+    scatter_nd_ref,
     attention_blockwise_ref,
     flash_decode_ref,
     split_kv_partials,

@@ -129,3 +129,16 @@ def combine_partials(o, m, l):
     big = m.max()
     w = torch.exp(m - big)
     return (w.unsqueeze(-1) * o).sum(dim=0) / (w * l).sum()
+
+
+def scatter_nd_ref(data, indices, updates):
+    """data[indices[i]] += updates[i] for every index row (duplicates accumulate), fp32 on the
+    CPU.  Restates what ke_scatter_nd computes (src/kernels/scatter_nd.cu:10-34) with the
+    library routine torch.Tensor.index_put_(accumulate=True)."""
+    out = data.detach().float().cpu().clone()
+    idx = indices.detach().cpu().long()
+    k = idx.shape[-1]
+    idx = idx.reshape(-1, k)
+    upd = updates.detach().float().cpu().reshape(idx.shape[0], *out.shape[k:])
+    out.index_put_(tuple(idx[:, j] for j in range(k)), upd, accumulate=True)
+    return out

@@ -91,7 +91,7 @@ def test_python_wrappers_validate_like_the_reference():
     # CPU tensors never reach a kernel: the op exists only for the CUDA dispatch key
     with pytest.raises((NotImplementedError, RuntimeError)):
         ops.gemm(t, t, torch.zeros(64, 64), 64, 64, 64, 1, 0)
-    assert sorted(ops.__all__) == ["FlashAttention", "flash_attention", "flash_decode", "fused_two_gemms", "gemm"]
+    assert sorted(ops.__all__) == ["FlashAttention", "flash_attention", "flash_decode", "fused_two_gemms", "gemm", "scatter_nd"]
 
 
 def test_op_schemas_match_the_reference():
@@ -99,6 +99,7 @@ def test_op_schemas_match_the_reference():
     import torch
     import tilefusion_amd  # noqa: F401
     want = {
+        "scatter_nd": "tilefusion::scatter_nd(Tensor data, Tensor(a!) updates, Tensor indices) -> ()",
         "gemm": "tilefusion::gemm(Tensor A, Tensor B, Tensor(a!) C, int m, int n, int k, int num_stages, int pipeline_level) -> ()",
         "fused_two_gemms": "tilefusion::fused_two_gemms(Tensor A, Tensor B, Tensor C, Tensor(a!) D, int tm, int tn, int tk, int tp) -> ()",
         "flash_attention": "tilefusion::flash_attention(Tensor Q, Tensor K, Tensor V, Tensor(a!) O, int tile_length_q, int tile_length_kv, int tile_hidden_qk, int tile_hidden_v, float softmax_scale, bool causal) -> ()",

@@ -123,3 +123,24 @@ def test_check_close_uses_contract_tolerances():
     assert N.check_close(ref + 5e-4, ref)[0]
     assert not N.check_close(ref + 5e-3, ref)[0]
     assert N.REL_L2_TOL == 1e-3 and N.MAX_ABS_TOL == 2e-2
+
+
+def test_scatter_nd_ref_matches_a_plain_loop():
+    # pins the index_put_ restatement: a dropped "accumulate", a transposed index or a wrong
+    # slice shape each fail this hand-written loop
+    g = torch.Generator().manual_seed(5)
+    data = torch.randn(3, 4, 5, generator=g)
+    idx = torch.tensor([[0, 1], [2, 3], [0, 1], [1, 0]])           # row 0 repeats
+    upd = torch.randn(4, 5, generator=g)
+    want = data.clone()
+    for i in range(idx.shape[0]):
+        for e in range(5):
+            want[idx[i, 0], idx[i, 1], e] += upd[i, e]
+    assert torch.allclose(N.scatter_nd_ref(data, idx, upd), want, atol=1e-6)
+    # index depth == rank: single elements
+    idx3 = torch.tensor([[0, 0, 0], [2, 3, 4], [0, 0, 0]])
+    upd3 = torch.tensor([1.0, 2.0, 4.0])
+    want = data.clone()
+    want[0, 0, 0] += 5.0
+    want[2, 3, 4] += 2.0
+    assert torch.allclose(N.scatter_nd_ref(data, idx3, upd3), want, atol=1e-6)

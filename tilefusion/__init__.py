@@ -7,7 +7,7 @@ import tilefusion_amd
 from tilefusion_amd import __version__, ops  # noqa: F401
 
 sys.modules[__name__ + ".ops"] = ops
-for _name in ("gemm", "fused_two_gemms", "flash_attention", "flash_decode"):
+for _name in ("gemm", "fused_two_gemms", "flash_attention", "flash_decode", "scatter_nd"):
     sys.modules[f"{__name__}.ops.{_name}"] = sys.modules[f"tilefusion_amd.ops.{_name}"]
 
 __all__ = ["ops"]

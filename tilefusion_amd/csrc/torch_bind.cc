@@ -168,6 +168,35 @@ void flash_decode(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V,
                "flash_decode");
 }
 
+// scatter_nd(data [d0..dr-1], updates [n.., d_k..d_{r-1}], indices [n.., k] int64): data[idx] += updates.
+// The reference's schema marks `updates` as the mutated tensor although its kernel writes
+// `data` (src/kernels/scatter_nd.cu:86-92); the schema is kept, `data` is what changes.
+void scatter_nd(const at::Tensor& data, at::Tensor& updates, const at::Tensor& indices) {
+  CHECK_INPUT(data);
+  CHECK_INPUT(updates);
+  CHECK_INPUT(indices);
+  TORCH_CHECK(indices.scalar_type() == at::kLong, "indices must be an int64 tensor.");
+  TORCH_CHECK(updates.scalar_type() == data.scalar_type(), "updates must have the dtype of data.");
+  TORCH_CHECK(data.dim() >= 1 && data.dim() <= 8 && indices.dim() >= 1, "scatter_nd: data rank must be 1..8.");
+  const int64_t k = indices.size(-1);
+  TORCH_CHECK(k >= 1 && k <= data.dim(), "scatter_nd: the last dimension of indices (", k,
+              ") must be within 1..rank of data (", data.dim(), ").");
+  const int64_t n = indices.numel() / k;
+  int64_t slice = 1;
+  for (int64_t i = k; i < data.dim(); ++i) slice *= data.size(i);
+  TORCH_CHECK(updates.numel() == n * slice, "scatter_nd: updates must hold ", n, " slices of ", slice,
+              " elements; got ", updates.numel(), " elements.");
+  int dtype = -1;
+  if (data.scalar_type() == at::kFloat) dtype = 0;
+  else if (data.scalar_type() == at::kHalf) dtype = 1;
+  else if (data.scalar_type() == at::kBFloat16) dtype = 2;
+  TORCH_CHECK(dtype >= 0, "scatter_nd: data must be float32, float16 or bfloat16.");
+  std::vector<int64_t> dims(data.sizes().begin(), data.sizes().end());
+  check_status(tf_scatter_nd(updates.data_ptr(), const_cast<at::Tensor&>(data).data_ptr(), indices.data_ptr<int64_t>(),
+                             dims.data(), (int)dims.size(), n, (int)k, dtype, current_stream()),
+               "scatter_nd");
+}
+
 }  // namespace kernels
 
 // Self-registering op table: each REGISTER_OP adds (schema, installer) at load time, and the
@@ -200,6 +229,7 @@ class KernelRegistry {
 #define REGISTER_OP(name, schema, func) \
   static const bool name##_registered = KernelRegistry::instance().add_kernel(#name, schema, func)
 
+REGISTER_OP(scatter_nd, "scatter_nd(Tensor data, Tensor(a!) updates, Tensor indices) -> ()", &kernels::scatter_nd);
 REGISTER_OP(gemm,
             "gemm(Tensor A, Tensor B, Tensor(a!) C, int m, int n, int k, "
             "int num_stages, int pipeline_level) -> ()",

@@ -4,6 +4,7 @@ from .flash_attention import FlashAttention, flash_attention
 from .flash_decode import flash_decode
 from .fused_two_gemms import fused_two_gemms
 from .gemm import gemm
+from .scatter_nd import scatter_nd
 
 __all__ = [
     "FlashAttention",
@@ -11,4 +12,5 @@ __all__ = [
     "flash_decode",
     "fused_two_gemms",
     "gemm",
+    "scatter_nd",
 ]
