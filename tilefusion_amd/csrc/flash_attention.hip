@@ -109,35 +109,41 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   // slice stream the same K/V through ONE L2 instead of eight.
   //   non-causal: items in slice-major order, cut into 8 contiguous chunks (the last one may
   //               be short; its surplus workgroups exit at once);
-  //   causal:     work per query tile varies 1..q_tiles, so every queue is sorted
-  //               heaviest (latest) tile first across the slices it owns; with a slice count
-  //               that is not a multiple of 8 the queues would be unequal, so the order falls
-  //               back to heaviest-first over all slices.
-  int qt;
+  //   causal:     work per query tile grows with its position, so a workgroup takes query
+  //               tile q_tiles-1-p and then tile p of the same slice: every workgroup does the
+  //               same amount of work, no sorting by weight is needed and the slice-major
+  //               order (with its L2 locality) is kept.  An odd number of query tiles falls
+  //               back to one tile per workgroup, heaviest tiles first over all slices.
+  int qt_of_pass[2] = {0, 0};
+  int num_passes = 1;
   size_t bh;
-  if (!kCausal) {
+  if (!kCausal || q_tiles % 2 == 0) {
+    const int per_slice = kCausal ? q_tiles / 2 : q_tiles;
     const int per_xcd = (total_items + 7) / 8;
     const int item = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
     if (item >= total_items) return;
-    qt = item % q_tiles;
-    bh = item / q_tiles;
+    const int p = item % per_slice;
+    bh = item / per_slice;
+    if (kCausal) {
+      qt_of_pass[0] = q_tiles - 1 - p;
+      qt_of_pass[1] = p;
+      num_passes = 2;
+    } else {
+      qt_of_pass[0] = p;
+    }
   } else {
     if ((int)blockIdx.x >= total_items) return;
     const int slices = total_items / q_tiles;
-    if (slices % 8 == 0) {
-      const int per = slices / 8, slot = blockIdx.x / 8;
-      qt = q_tiles - 1 - slot / per;
-      bh = (blockIdx.x % 8) * per + slot % per;
-    } else {
-      qt = q_tiles - 1 - (int)blockIdx.x / slices;
-      bh = blockIdx.x % slices;
-    }
+    qt_of_pass[0] = q_tiles - 1 - (int)blockIdx.x / slices;
+    bh = blockIdx.x % slices;
   }
   Q += bh * (size_t)Lq * D;
   K += bh * (size_t)Lkv * D;
   V += bh * (size_t)Lkv * DV;
   O += bh * (size_t)Lq * DV;
 
+  for (int pass = 0; pass < num_passes; ++pass) {
+  const int qt = qt_of_pass[pass];
   const int q_row0 = qt * kBMq + wave * kRowsPerWave;  // first query row of this wavefront
   // this lane's query rows: block qb holds row q_row0 + 16*qb + lr
 
@@ -464,6 +470,9 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       }
     }
   }
+  // the next pass re-fills the ring: nobody may still be reading the last tiles
+  if (pass + 1 < num_passes) __syncthreads();
+  }  // pass
 }
 
 template <int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQB>
@@ -476,7 +485,8 @@ int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, in
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
   constexpr int bm = kWavesT * 16 * kQB;
   const int q_tiles = (Lq + bm - 1) / bm;
-  const int total_items = q_tiles * batch;
+  // causal with an even tile count: one workgroup per PAIR of query tiles (see the kernel)
+  const int total_items = (kCausal && q_tiles % 2 == 0) ? (q_tiles / 2) * batch : q_tiles * batch;
   const dim3 grid(8 * ((total_items + 7) / 8));
   hipLaunchKernelGGL(kern, grid, dim3(kWavesT * 64), lds, st,
                      static_cast<const half_t*>(Q), static_cast<const half_t*>(K),
