@@ -4,10 +4,11 @@
 import sys
 
 import tilefusion_amd
-from tilefusion_amd import __version__, ops  # noqa: F401
+from tilefusion_amd import __version__, jit, ops  # noqa: F401
 
 sys.modules[__name__ + ".ops"] = ops
+sys.modules[__name__ + ".jit"] = jit
 for _name in ("gemm", "fused_two_gemms", "flash_attention", "flash_decode", "scatter_nd"):
     sys.modules[f"{__name__}.ops.{_name}"] = sys.modules[f"tilefusion_amd.ops.{_name}"]
 
-__all__ = ["ops"]
+__all__ = ["jit", "ops"]
