@@ -236,6 +236,50 @@ TT_API int tt_readme_gemm(const void* a, const void* b, void* c) {
   return launch_status();
 }
 
+// ---- 3b. the same GEMM with the other MMA atoms: bf16 inputs, and fp16 inputs with an fp16
+//          accumulator tile (include/cell/compute/gemm.hpp:63-150 in the reference) -------------
+namespace atoms {
+template <typename InType, typename AccType>
+__global__ void gemm_atom(const InType* dA, const InType* dB, AccType* dC) {
+  using WarpLayout = tl::RowMajor<2, 2>;
+  constexpr int kM = 128, kN = 64, kK = 256, kTK = 32;
+  using GlobalA = GlobalTile<InType, tl::RowMajor<kM, kK>>;
+  using IteratorA = TileIterator<GlobalA, TileShape<kM, kTK>>;
+  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kM / 2 / 16, kTK / 32>>;
+  using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kN>>;
+  using IteratorB = TileIterator<GlobalB, TileShape<kTK, kN>>;
+  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kN / 2 / 16>>;
+  using GlobalC = GlobalTile<AccType, tl::RowMajor<kM, kN>>;
+  using RegC = RegTile<BaseTileAccRowMajor<AccType>, tl::RowMajor<kM / 2 / 16, kN / 2 / 16>>;
+  IteratorA gAs(dA);
+  IteratorB gBs(dB);
+  RegA rA;
+  RegB rB;
+  RegC acc;
+  GlobalToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont> loader_a;
+  GlobalToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont> loader_b;
+  for (int k = 0; k < IteratorA::sc1; ++k) {
+    loader_a(gAs(k), rA);
+    loader_b(gBs(k), rB);
+    compute::gemm(rA, rB, acc);
+  }
+  GlobalC gC(dC);
+  RegToGlobalStorer<GlobalC, RegC, WarpLayout> storer_c;
+  storer_c(acc, gC);
+}
+}  // namespace atoms
+TT_API int tt_atom_gemm(int variant, const void* a, const void* b, void* c) {
+  if (variant == 0)
+    hipLaunchKernelGGL((atoms::gemm_atom<__bfloat16, float>), dim3(1), dim3(256), 0, 0, static_cast<const __bfloat16*>(a),
+                       static_cast<const __bfloat16*>(b), static_cast<float*>(c));
+  else if (variant == 1)
+    hipLaunchKernelGGL((atoms::gemm_atom<__half, __half>), dim3(1), dim3(256), 0, 0, static_cast<const __half*>(a),
+                       static_cast<const __half*>(b), static_cast<__half*>(c));
+  else
+    return -1;
+  return launch_status();
+}
+
 // ---- 4. ke_gemm composed from the primitives (test_gemm.cu:172-215,316-375) ------------------
 template <typename Traits, typename AccType>
 __global__ void k_ke_gemm(const __half* a, const __half* b, AccType* c) {

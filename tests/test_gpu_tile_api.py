@@ -36,6 +36,7 @@ def lib():
     lib.tt_swizzled_fragments.argtypes = [_i, _vp, _vp, _vp]
     lib.tt_acc_roundtrip.argtypes = [_i, _vp, _vp, _vp, _vp]
     lib.tt_readme_gemm.argtypes = [_vp, _vp, _vp]
+    lib.tt_atom_gemm.argtypes = [_i, _vp, _vp, _vp]
     lib.tt_ke_gemm.argtypes = [_i, _vp, _vp, _vp]
     lib.tt_ke_gemm_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 4
     lib.tt_softmax_pieces.argtypes = [_i, _vp, _vp, _vp, _vp, _i, _i]
@@ -91,6 +92,21 @@ def test_readme_example_gemm(lib):
     b = torch.randint(-3, 4, (64, 256), generator=g).half()
     assert lib.tt_readme_gemm(a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.data_ptr()) == 0
     assert torch.equal(c.cpu(), N.gemm_ref(a, b))
+
+
+def test_other_mma_atoms(lib):
+    # bf16 x bf16 -> fp32, and fp16 x fp16 with an fp16 accumulator tile (rounded once per atom)
+    a, b = oracle.make_c1_gemm_inputs()
+    ref = N.gemm_ref(a.bfloat16(), b.bfloat16())
+    c = torch.full((128, 64), float("nan"), device=DEV)
+    assert lib.tt_atom_gemm(0, a.bfloat16().to(DEV).data_ptr(), b.bfloat16().to(DEV).data_ptr(), c.data_ptr()) == 0
+    ok, r, m = N.check_close(c, ref)
+    assert ok and m < 1e-4, (r, m)
+    ch = torch.full((128, 64), float("nan"), device=DEV, dtype=torch.float16)
+    assert lib.tt_atom_gemm(1, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), ch.data_ptr()) == 0
+    ref = N.gemm_ref(a, b)
+    # 8 roundings to fp16 along K = 256 (one per 32-deep atom): a few fp16 ulps of |C| ~ 10
+    assert N.rel_l2(ch, ref) <= 2e-3 and N.max_abs(ch, ref) <= 5e-2, (N.rel_l2(ch, ref), N.max_abs(ch, ref))
 
 
 @pytest.mark.parametrize("variant", range(6))

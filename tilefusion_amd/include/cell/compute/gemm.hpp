@@ -53,6 +53,28 @@ struct MmaAtom<__bfloat16, __bfloat16, float, MMA_ATOM_16x16x32> {
   }
 };
 
+// fp16 accumulator tile (counterpart of MmaAtom<__half, __half, __half>, include/cell/compute/
+// gemm.hpp:63-105).  CDNA4 has no MFMA that accumulates in fp16: the product is accumulated in
+// fp32 by the same instruction and rounded to fp16 once per atom, which is at least as
+// accurate as the reference's fp16-accumulating mma.sync.
+template <>
+struct MmaAtom<__half, __half, __half, MMA_ATOM_16x16x32> {
+  using BaseTileA = BaseTileRowMajor<__half>;
+  using BaseTileB = BaseTileColMajor<__half>;
+  using BaseTileC = BaseTileAccRowMajor<__half>;
+  using BaseTile = BaseTileShape<__half>;
+  DEVICE void operator()(const BaseTileA& a, const BaseTileB& b, BaseTileC& c) const {
+    const auto va = *reinterpret_cast<const detail::half8_v*>(a.data());
+    const auto vb = *reinterpret_cast<const detail::half8_v*>(b.data());
+    detail::float4_v vc;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) vc[r] = to_float(c.data()[r]);
+    vc = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, vb, vc, 0, 0, 0);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) c.mutable_data()[r] = from_float<__half>(vc[r]);
+  }
+};
+
 template <typename RegTileA, typename RegTileB, typename RegTileC, typename AtomicShape = MMA_ATOM_16x16x16>
 struct Gemm {
   using InTypeA = typename RegTileA::DType::DType;
