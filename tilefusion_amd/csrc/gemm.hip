@@ -313,6 +313,190 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
+// 256 x 256 x 64 path: same 2 x 2 wavefronts of 128 x 128, but k-tiles of 64 so that every
+// global->LDS instruction fetches whole 128-byte lines (8 rows x 128 bytes).  The vector L1
+// moves full lines, so the 64-byte row segments of a 32-deep tile spend half of the L2->L1
+// bandwidth on bytes that are dropped and requested again one k-tile later.
+//
+// A 64-deep tile is 64 KiB and only 160 KiB of LDS exist, so the ring is kept in UNITS of one
+// operand of one tile (32 KiB, five of them): unit u lives in ring slot u % 5, A of tile t is
+// unit 2t and B of tile t unit 2t+1.  Iteration t:
+//   k-step 0: multiplies fragments (t, 0), reads fragments (t, 1), requests A of tile t+2 into
+//             the slot B of tile t-1 left;
+//   barrier:  tile t is read out (both its units are free) and tile t+1 has landed
+//             (vmcnt leaves only the 8 requests of k-step 0 outstanding);
+//   k-step 1: multiplies (t, 1), reads fragments (t+1, 0), requests B of tile t+2 into the
+//             slot A of tile t left.
+// Every request has at least 8 MFMA slots (1024 MFMA cycles) to land, as in the 4-stage ring.
+// ------------------------------------------------------------------------------------------
+struct Ring64Shape {
+  static constexpr int BM = 256, BN = 256, BK = 64;
+  static constexpr int kWaves = 4, kThreads = 256;
+  static constexpr int WM = 128, WN = 128, TM = 8, TN = 8;
+  static constexpr int kRowBytes = BK * 2;                 // 128
+  static constexpr int kUnitBytes = BM * kRowBytes;        // 32 KiB: one operand of one tile
+  static constexpr int kUnits = 5;
+  static constexpr int kLoads = BM / 8 / kWaves;           // 1 KiB requests per wavefront and unit
+  // 128-byte rows: two rows per pass over the banks; chunk ^ (row / 2) % 8 keeps every
+  // ds_read_b128 lane pass on 16 different bank groups
+  __host__ __device__ static constexpr int swizzle(int row, int c) { return c ^ ((row / 2) % 8); }
+};
+
+#ifndef TFK_GEMM_R64_FIRST
+#define TFK_GEMM_R64_FIRST 8   // slots of a k-step over which its unit's 8 requests are spread
+#endif
+
+template <typename OutT>
+__global__ __launch_bounds__(Ring64Shape::kThreads) void gemm_ring64_kernel(
+    const half_t* __restrict__ A, const half_t* __restrict__ B, OutT* __restrict__ C, int M,
+    int N, int K, int tiles_m, int tiles_n) {
+  using S = Ring64Shape;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int tile_m, tile_n;
+  tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
+  const int m0 = tile_m * S::BM, n0 = tile_n * S::BN;
+  const int wm = wave / 2, wn = wave % 2;
+
+  // global -> LDS plan: request n of a wavefront covers rows (wave + 4n) * 8 .. +7 of a unit;
+  // lane l fills physical chunk l % 8 of row l / 8 and fetches the logical chunk the swizzle
+  // maps there.  A and B share the per-lane offsets (same row stride K).
+  const int ld_row = wave * 8 + lane / 8, ld_c = lane % 8;
+  const char* a_tile = reinterpret_cast<const char*>(A + (size_t)m0 * K);
+  const char* b_tile = reinterpret_cast<const char*>(B + (size_t)n0 * K);
+  unsigned g_off[S::kLoads];
+#pragma unroll
+  for (int n = 0; n < S::kLoads; ++n)
+    g_off[n] = (unsigned)(ld_row + 32 * n) * (unsigned)K * 2u + (unsigned)S::swizzle(ld_row, ld_c) * 16u;
+  // LDS -> fragment plan: fragment i of k-step ks: row 16*i + l%16 of the wavefront's 128,
+  // logical chunk 4*ks + l/16
+  const int fr = lane & 15, fg = lane >> 4;
+  unsigned a_rd[2], b_rd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks) {
+    a_rd[ks] = (wm * S::WM + fr) * S::kRowBytes + S::swizzle(fr, 4 * ks + fg) * 16;
+    b_rd[ks] = (wn * S::WN + fr) * S::kRowBytes + S::swizzle(fr, 4 * ks + fg) * 16;
+  }
+
+  float4_t acc[S::TM][S::TN];
+#pragma unroll
+  for (int i = 0; i < S::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < S::TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int num_k_tiles = K / S::BK;
+  // Slot i of a k-step multiplies A fragment i with all B fragments: B needs two full sets,
+  // A fragment i is dead once slot i has issued and is replaced in place by the next k-step's.
+  half8_t af[S::TM], bf[2][S::TN];
+  auto request = [&](const char* tile, int slot, int t, int n) __attribute__((always_inline)) {
+    const size_t kbyte = (size_t)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
+    load_global_to_lds_16B(tile + kbyte + g_off[n], smem + slot * S::kUnitBytes + (wave + 4 * n) * 1024);
+  };
+  auto frag_part = [&](int slot_a, int slot_b, int ks, int nbuf, int i) __attribute__((always_inline)) {
+    const char* ua = smem + slot_a * S::kUnitBytes;
+    const char* ub = smem + slot_b * S::kUnitBytes;
+    if (i < S::TN / 2) {
+      bf[nbuf][2 * i] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks] + (2 * i) * 16 * S::kRowBytes);
+      bf[nbuf][2 * i + 1] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks] + (2 * i + 1) * 16 * S::kRowBytes);
+    }
+    af[i] = *reinterpret_cast<const half8_t*>(ua + a_rd[ks] + i * 16 * S::kRowBytes);
+  };
+  auto mfma_slot = [&](int buf, int i) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma_16x16x32(bf[buf][j], af[i], acc[i][j]);
+  };
+  constexpr int kFirst = TFK_GEMM_R64_FIRST;
+  constexpr int kPerSlot = S::kLoads / kFirst;
+  static_assert(kPerSlot * kFirst == S::kLoads, "requests must split evenly over the slots");
+
+  // prologue: tiles 0 and 1 into ring slots 0..3; fragments (0, 0) once tile 0 is there
+#pragma unroll
+  for (int n = 0; n < S::kLoads; ++n) request(a_tile, 0, 0, n);
+#pragma unroll
+  for (int n = 0; n < S::kLoads; ++n) request(b_tile, 1, 0, n);
+#pragma unroll
+  for (int n = 0; n < S::kLoads; ++n) request(a_tile, 2, 1, n);
+#pragma unroll
+  for (int n = 0; n < S::kLoads; ++n) request(b_tile, 3, 1, n);
+  barrier_keep_vmem<2 * S::kLoads>();
+#pragma unroll
+  for (int i = 0; i < S::TM; ++i) frag_part(0, 1, 0, 0, i);
+
+  int sa = 0;   // ring slot of A of tile t; B of tile t is sa+1, A of t+1 sa+2, ... (mod 5)
+  auto ring = [](int s) __attribute__((always_inline)) { return s >= S::kUnits ? s - S::kUnits : s; };
+  for (int t = 0; t < num_k_tiles; ++t) {
+    const int sb = ring(sa + 1), sa1 = ring(sa + 2), sb1 = ring(sa + 3), sa2 = ring(sa + 4);
+#pragma unroll
+    for (int i = 0; i < S::TM; ++i) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (i < kFirst) {
+#pragma unroll
+        for (int n = i * kPerSlot; n < (i + 1) * kPerSlot; ++n) request(a_tile, sa2, t + 2, n);
+      }
+      mfma_slot(0, i);
+      frag_part(sa, sb, 1, 1, i);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    barrier_keep_vmem<S::kLoads>();
+#pragma unroll
+    for (int i = 0; i < S::TM; ++i) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (i < kFirst) {
+#pragma unroll
+        for (int n = i * kPerSlot; n < (i + 1) * kPerSlot; ++n) request(b_tile, sa, t + 2, n);
+      }
+      mfma_slot(1, i);
+      frag_part(sa1, sb1, 0, 0, i);
+    }
+    sa = sa1;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  wait_vmem_all();  // the clamped tail requests must not outlive the workgroup's LDS
+
+  // --- epilogue (same accumulator layout as the 32-deep kernel) -----------------------------
+  const int c_row0 = m0 + wm * S::WM + fr;
+  const int c_col0 = n0 + wn * S::WN + 4 * fg;
+#pragma unroll
+  for (int i = 0; i < S::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < S::TN; ++j) {
+      OutT* dst = C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j;
+      if constexpr (sizeof(OutT) == 2) {
+        half4_t v;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][r];
+        *reinterpret_cast<half4_t*>(dst) = v;
+      } else {
+        *reinterpret_cast<float4_t*>(dst) = acc[i][j];
+      }
+    }
+}
+
+template <typename OutT>
+int launch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
+  using S = Ring64Shape;
+  auto kern = gemm_ring64_kernel<OutT>;
+  constexpr int lds = S::kUnits * S::kUnitBytes;
+  static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
+  static thread_local int configured_dev = -1;
+  int dev = 0;
+  TFK_HIP_TRY(hipGetDevice(&dev));
+  if (configured_dev != dev) {
+    TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    configured_dev = dev;
+  }
+  const int tiles_m = M / S::BM, tiles_n = N / S::BN;
+  hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(S::kThreads), lds, st,
+                     static_cast<const half_t*>(A), static_cast<const half_t*>(B),
+                     static_cast<OutT*>(C), M, N, K, tiles_m, tiles_n);
+  TFK_HIP_TRY(hipGetLastError());
+  return TF_OK;
+}
+
+// ------------------------------------------------------------------------------------------
 // General path: any M, N; K % 8 == 0.  Register-staged, bounds-checked, one LDS stage.
 // ------------------------------------------------------------------------------------------
 template <typename S, typename OutT>
@@ -425,6 +609,10 @@ int launch_guarded(const void* A, const void* B, void* C, int M, int N, int K, h
 
 template <typename OutT>
 int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
+#ifndef TFK_GEMM_NO_RING64
+  if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
+    return launch_ring64<OutT>(A, B, C, M, N, K, st);
+#endif
   if (M % 256 == 0 && N % 256 == 0 && K % ShapeBig::BK == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
     return launch_direct<ShapeBig, OutT>(A, B, C, M, N, K, st);
   if (M % 128 == 0 && N % 128 == 0 && K % 32 == 0)
