@@ -329,28 +329,47 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
 //             slot A of tile t left.
 // Every request has at least 8 MFMA slots (1024 MFMA cycles) to land, as in the 4-stage ring.
 // ------------------------------------------------------------------------------------------
+template <int WAVES_N_>
 struct Ring64Shape {
   static constexpr int BM = 256, BN = 256, BK = 64;
-  static constexpr int kWaves = 4, kThreads = 256;
-  static constexpr int WM = 128, WN = 128, TM = 8, TN = 8;
-  static constexpr int kRowBytes = BK * 2;                 // 128
-  static constexpr int kUnitBytes = BM * kRowBytes;        // 32 KiB: one operand of one tile
+  static constexpr int WAVES_M = 2, WAVES_N = WAVES_N_;
+  static constexpr int kWaves = WAVES_M * WAVES_N, kThreads = kWaves * kWaveSize;
+  static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  static constexpr int TM = WM / 16, TN = WN / 16;          // 16x16 MFMA tiles per wavefront
+  static constexpr int kRowBytes = BK * 2;                  // 128
+  static constexpr int kUnitBytes = BM * kRowBytes;         // 32 KiB: one operand of one tile
   static constexpr int kUnits = 5;
-  static constexpr int kLoads = BM / 8 / kWaves;           // 1 KiB requests per wavefront and unit
+  static constexpr int kLoads = BM / 8 / kWaves;            // 1 KiB requests per wavefront and unit
+  static_assert(TM == 8 && (TN == 8 || TN == 4) && TM % kLoads == 0, "slot schedule assumes 8 slots per k-step");
   // 128-byte rows: two rows per pass over the banks; chunk ^ (row / 2) % 8 keeps every
   // ds_read_b128 lane pass on 16 different bank groups
-  __host__ __device__ static constexpr int swizzle(int row, int c) { return c ^ ((row / 2) % 8); }
+#ifndef TFK_R64_SWZ
+#define TFK_R64_SWZ 0
+#endif
+  __host__ __device__ static constexpr int swizzle(int row, int c) {
+    if (TFK_R64_SWZ == 1) return c ^ (((row / 2) % 4) << 1);   // 32-byte pairs stay in order
+    if (TFK_R64_SWZ == 2) return c ^ (((row / 2) % 2) << 2);   // 64-byte halves stay in order
+    if (TFK_R64_SWZ == 3) return c;
+    return c ^ ((row / 2) % 8);
+  }
 };
 
-#ifndef TFK_GEMM_R64_FIRST
-#define TFK_GEMM_R64_FIRST 8   // slots of a k-step over which its unit's 8 requests are spread
+#ifndef TFK_R64_PLAIN_MFMA
+#define TFK_R64_ASM_MFMA
+#endif
+#ifndef TFK_R64_RD_POS
+#define TFK_R64_RD_POS 1
+#endif
+#if defined(TFK_R64_NOREQ)   // timing experiments only: results are wrong without the requests
+#define TFK_R64_REQUEST(...)
+#else
+#define TFK_R64_REQUEST(...) request(__VA_ARGS__)
 #endif
 
-template <typename OutT>
-__global__ __launch_bounds__(Ring64Shape::kThreads) void gemm_ring64_kernel(
+template <typename S, typename OutT>
+__global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     const half_t* __restrict__ A, const half_t* __restrict__ B, OutT* __restrict__ C, int M,
     int N, int K, int tiles_m, int tiles_n) {
-  using S = Ring64Shape;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -358,19 +377,21 @@ __global__ __launch_bounds__(Ring64Shape::kThreads) void gemm_ring64_kernel(
   int tile_m, tile_n;
   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * S::BM, n0 = tile_n * S::BN;
-  const int wm = wave / 2, wn = wave % 2;
+  const int wm = wave / S::WAVES_N, wn = wave % S::WAVES_N;
 
-  // global -> LDS plan: request n of a wavefront covers rows (wave + 4n) * 8 .. +7 of a unit;
-  // lane l fills physical chunk l % 8 of row l / 8 and fetches the logical chunk the swizzle
-  // maps there.  A and B share the per-lane offsets (same row stride K).
+  // global -> LDS plan: request n of a wavefront covers rows (wave + kWaves*n) * 8 .. +7 of a
+  // unit; lane l fills physical chunk l % 8 of row l / 8 and fetches the logical chunk the
+  // swizzle maps there.  A and B share the per-lane offsets (same row stride K); the address
+  // is a scalar base (tile origin + k offset) plus this 32-bit per-lane offset, so a request
+  // needs no vector arithmetic.
   const int ld_row = wave * 8 + lane / 8, ld_c = lane % 8;
   const char* a_tile = reinterpret_cast<const char*>(A + (size_t)m0 * K);
   const char* b_tile = reinterpret_cast<const char*>(B + (size_t)n0 * K);
   unsigned g_off[S::kLoads];
 #pragma unroll
   for (int n = 0; n < S::kLoads; ++n)
-    g_off[n] = (unsigned)(ld_row + 32 * n) * (unsigned)K * 2u + (unsigned)S::swizzle(ld_row, ld_c) * 16u;
-  // LDS -> fragment plan: fragment i of k-step ks: row 16*i + l%16 of the wavefront's 128,
+    g_off[n] = (unsigned)(ld_row + 8 * S::kWaves * n) * (unsigned)K * 2u + (unsigned)S::swizzle(ld_row, ld_c) * 16u;
+  // LDS -> fragment plan: fragment i of k-step ks: row 16*i + l%16 of the wavefront's rows,
   // logical chunk 4*ks + l/16
   const int fr = lane & 15, fg = lane >> 4;
   unsigned a_rd[2], b_rd[2];
@@ -387,19 +408,54 @@ __global__ __launch_bounds__(Ring64Shape::kThreads) void gemm_ring64_kernel(
     for (int j = 0; j < S::TN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   const int num_k_tiles = K / S::BK;
+  const unsigned smem_addr = lds_address(smem);
   // Slot i of a k-step multiplies A fragment i with all B fragments: B needs two full sets,
   // A fragment i is dead once slot i has issued and is replaced in place by the next k-step's.
   half8_t af[S::TM], bf[2][S::TN];
+  // The requests are issued from inline assembly: the compiler then keeps exact counts for the
+  // fragment reads (a direct-to-LDS load it knows about makes every LDS wait a full drain),
+  // and the vector-memory waits are placed by hand below.
+#ifdef TFK_R64_BUFFER
+  typedef int rsrc_t __attribute__((ext_vector_type(4)));
+  auto make_rsrc = [](const char* base) __attribute__((always_inline)) {
+    const unsigned long long a = (unsigned long long)base;
+    rsrc_t r;
+    r[0] = __builtin_amdgcn_readfirstlane((int)(a & 0xffffffffu));
+    r[1] = __builtin_amdgcn_readfirstlane((int)(a >> 32));
+    r[2] = (int)0xffffffffu;
+    r[3] = 0x00020000;
+    return r;
+  };
+  const rsrc_t a_rsrc = make_rsrc(a_tile), b_rsrc = make_rsrc(b_tile);
+  auto request = [&](const char* tile, int slot, int t, int n) __attribute__((always_inline)) {
+    const unsigned kbyte = (unsigned)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
+    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+                 :
+                 : "v"(g_off[n]), "s"(tile == a_tile ? a_rsrc : b_rsrc), "s"(kbyte),
+                   "s"(smem_addr + slot * S::kUnitBytes + (wave + S::kWaves * n) * 1024)
+                 : "memory");
+  };
+#else
   auto request = [&](const char* tile, int slot, int t, int n) __attribute__((always_inline)) {
     const size_t kbyte = (size_t)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
-    load_global_to_lds_16B(tile + kbyte + g_off[n], smem + slot * S::kUnitBytes + (wave + 4 * n) * 1024);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(g_off[n]), "s"(tile + kbyte),
+                   "s"(smem_addr + slot * S::kUnitBytes + (wave + S::kWaves * n) * 1024)
+                 : "memory");
   };
+#endif
+  // Fragment requests of slot i for the NEXT k-step: the B fragments in the first slots (two
+  // per slot at TN = 8, one at TN = 4; all of them are needed by the next k-step's slot 0),
+  // then its own A fragment.
+  constexpr int kBPerSlot = S::TN / 4;
   auto frag_part = [&](int slot_a, int slot_b, int ks, int nbuf, int i) __attribute__((always_inline)) {
     const char* ua = smem + slot_a * S::kUnitBytes;
     const char* ub = smem + slot_b * S::kUnitBytes;
-    if (i < S::TN / 2) {
-      bf[nbuf][2 * i] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks] + (2 * i) * 16 * S::kRowBytes);
-      bf[nbuf][2 * i + 1] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks] + (2 * i + 1) * 16 * S::kRowBytes);
+    if (i < 4) {
+#pragma unroll
+      for (int f = kBPerSlot * i; f < kBPerSlot * (i + 1); ++f)
+        bf[nbuf][f] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks] + f * 16 * S::kRowBytes);
     }
     af[i] = *reinterpret_cast<const half8_t*>(ua + a_rd[ks] + i * 16 * S::kRowBytes);
   };
@@ -407,22 +463,96 @@ __global__ __launch_bounds__(Ring64Shape::kThreads) void gemm_ring64_kernel(
 #pragma unroll
     for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma_16x16x32(bf[buf][j], af[i], acc[i][j]);
   };
-  constexpr int kFirst = TFK_GEMM_R64_FIRST;
-  constexpr int kPerSlot = S::kLoads / kFirst;
-  static_assert(kPerSlot * kFirst == S::kLoads, "requests must split evenly over the slots");
+  // Issue order inside a slot: the fragment reads go between the MFMAs, one at a time (a
+  // 16-cycle MFMA leaves room for one LDS instruction behind it; a cluster of reads stalls the
+  // matrix pipe).  The request sits at the slot boundary.
+  auto interleave = [&](int i) __attribute__((always_inline)) {
+    if constexpr (S::TN == 8) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (i < 4) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+      }
+    } else {
+      if (i < 4) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      } else {
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      }
+    }
+  };
+#ifdef TFK_R64_ASM_MFMA
+  // Slot with the MFMAs issued from inline assembly, accumulators pinned to AGPRs, and the
+  // slot's fragment reads placed by hand between them.
+  half8_t afx[2][S::TM];
+  auto slot_pinned = [&](int buf, int i, int slot_a, int slot_b, int ks_next) __attribute__((always_inline)) {
+    const char* ua = smem + slot_a * S::kUnitBytes;
+    const char* ub = smem + slot_b * S::kUnitBytes;
+    constexpr int kReadsB = S::TN / 4;            // B fragments fetched by slots 0..3
+    const int n_reads = (i < 4 ? kReadsB : 0) + 1;
+    int done = 0;
+#pragma unroll
+    for (int j = 0; j < S::TN; ++j) {
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bf[buf][j]), "v"(afx[buf][i]));
+      // after MFMA j: issue read number `done` if j hits its position (spread evenly)
+      if (done < n_reads && j == (done * S::TN) / n_reads + TFK_R64_RD_POS) {
+        __builtin_amdgcn_sched_barrier(0);
+        if (i < 4 && done < kReadsB) {
+          const int f = kReadsB * i + done;
+          bf[buf ^ 1][f] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks_next] + f * 16 * S::kRowBytes);
+        } else {
+          afx[buf ^ 1][i] = *reinterpret_cast<const half8_t*>(ua + a_rd[ks_next] + i * 16 * S::kRowBytes);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        ++done;
+      }
+    }
+  };
+#endif
+  // Workgroup barrier that keeps the youngest kLoads requests in flight.  The LDS wait and the
+  // barrier are builtins so that the compiler knows every earlier fragment read has returned.
+  auto ring_barrier = [&]() __attribute__((always_inline)) {
+    wait_vmem<S::kLoads>();
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  constexpr int kSlotsPerLoad = S::TM / S::kLoads;   // a request every so many slots
 
   // prologue: tiles 0 and 1 into ring slots 0..3; fragments (0, 0) once tile 0 is there
 #pragma unroll
-  for (int n = 0; n < S::kLoads; ++n) request(a_tile, 0, 0, n);
+  for (int u = 0; u < 4; ++u)
 #pragma unroll
-  for (int n = 0; n < S::kLoads; ++n) request(b_tile, 1, 0, n);
+    for (int n = 0; n < S::kLoads; ++n) request(u % 2 ? b_tile : a_tile, u, u / 2, n);
+  wait_vmem<2 * S::kLoads>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+#ifdef TFK_R64_ASM_MFMA
 #pragma unroll
-  for (int n = 0; n < S::kLoads; ++n) request(a_tile, 2, 1, n);
+  for (int f = 0; f < S::TN; ++f)
+    bf[0][f] = *reinterpret_cast<const half8_t*>(smem + S::kUnitBytes + b_rd[0] + f * 16 * S::kRowBytes);
 #pragma unroll
-  for (int n = 0; n < S::kLoads; ++n) request(b_tile, 3, 1, n);
-  barrier_keep_vmem<2 * S::kLoads>();
+  for (int i = 0; i < S::TM; ++i)
+    afx[0][i] = *reinterpret_cast<const half8_t*>(smem + a_rd[0] + i * 16 * S::kRowBytes);
+#else
 #pragma unroll
   for (int i = 0; i < S::TM; ++i) frag_part(0, 1, 0, 0, i);
+#endif
 
   int sa = 0;   // ring slot of A of tile t; B of tile t is sa+1, A of t+1 sa+2, ... (mod 5)
   auto ring = [](int s) __attribute__((always_inline)) { return s >= S::kUnits ? s - S::kUnits : s; };
@@ -431,53 +561,94 @@ __global__ __launch_bounds__(Ring64Shape::kThreads) void gemm_ring64_kernel(
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i < kFirst) {
-#pragma unroll
-        for (int n = i * kPerSlot; n < (i + 1) * kPerSlot; ++n) request(a_tile, sa2, t + 2, n);
-      }
+      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(a_tile, sa2, t + 2, i / kSlotsPerLoad);
+#ifdef TFK_R64_ASM_MFMA
+      slot_pinned(0, i, sa, sb, 1);
+#else
       mfma_slot(0, i);
       frag_part(sa, sb, 1, 1, i);
+      interleave(i);
+#endif
     }
     __builtin_amdgcn_sched_barrier(0);
-    barrier_keep_vmem<S::kLoads>();
+    ring_barrier();
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i < kFirst) {
-#pragma unroll
-        for (int n = i * kPerSlot; n < (i + 1) * kPerSlot; ++n) request(b_tile, sa, t + 2, n);
-      }
+      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(b_tile, sa, t + 2, i / kSlotsPerLoad);
+#ifdef TFK_R64_ASM_MFMA
+      slot_pinned(1, i, sa1, sb1, 0);
+#else
       mfma_slot(1, i);
       frag_part(sa1, sb1, 0, 0, i);
+      interleave(i);
+#endif
     }
     sa = sa1;
+#ifdef TFK_R64_ASM_MFMA
+    // The compiler does not know that the accumulators are written by MFMAs (they are issued
+    // from assembly), so nothing would keep it from reading the youngest results right behind
+    // the loop without the wait states the matrix pipe needs.  The delay therefore sits inside
+    // the last iteration, in front of anything the register allocator may put on the exit
+    // edge.  The iteration count is laundered through an empty asm so that the test is not
+    // recognised as the exit condition and sunk out of the loop.
+    int t_seen = t;
+    asm volatile("" : "+s"(t_seen));
+    if (t_seen + 1 == num_k_tiles) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#endif
   }
   __builtin_amdgcn_sched_barrier(0);
   wait_vmem_all();  // the clamped tail requests must not outlive the workgroup's LDS
-
-  // --- epilogue (same accumulator layout as the 32-deep kernel) -----------------------------
+  // --- epilogue -----------------------------------------------------------------------------
+  // acc[i][j][r] = C[.. + 16*i + l%16][.. + 16*j + 4*(l/16) + r].  For fp16 output the lanes of
+  // 16-lane groups g and g^1 trade halves of a pair of tiles (v_permlane16_swap): group g even
+  // ends up with 8 consecutive columns of tile j, group g odd with 8 of tile j+1, so every lane
+  // stores 16 bytes and four lanes cover 64 contiguous bytes of a row (8-byte stores cost the
+  // address unit four times as many accesses for the same data).
   const int c_row0 = m0 + wm * S::WM + fr;
-  const int c_col0 = n0 + wn * S::WN + 4 * fg;
+  if constexpr (sizeof(OutT) == 2) {
+    const int c_col0 = n0 + wn * S::WN + 16 * (fg & 1) + 4 * (fg & 2);
 #pragma unroll
-  for (int i = 0; i < S::TM; ++i)
+    for (int i = 0; i < S::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < S::TN; ++j) {
-      OutT* dst = C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j;
-      if constexpr (sizeof(OutT) == 2) {
-        half4_t v;
+      for (int j = 0; j < S::TN; j += 2) {
+        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+        unsigned x[2], y[2];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][r];
-        *reinterpret_cast<half4_t*>(dst) = v;
-      } else {
-        *reinterpret_cast<float4_t*>(dst) = acc[i][j];
+        for (int d = 0; d < 2; ++d) {
+          const h2_t hx = {(half_t)acc[i][j][2 * d], (half_t)acc[i][j][2 * d + 1]};
+          const h2_t hy = {(half_t)acc[i][j + 1][2 * d], (half_t)acc[i][j + 1][2 * d + 1]};
+          x[d] = __builtin_bit_cast(unsigned, hx);
+          y[d] = __builtin_bit_cast(unsigned, hy);
+#if defined(__HIP_DEVICE_COMPILE__)
+          // odd groups receive x of the group below into x; even groups receive y ... see above:
+          // swap(x, y): x of odd groups <-> y of even groups
+          auto sw = __builtin_amdgcn_permlane16_swap(x[d], y[d], false, false);
+          x[d] = sw[0];
+          y[d] = sw[1];
+#endif
+        }
+        uint4_t v = {x[0], x[1], y[0], y[1]};
+        *reinterpret_cast<uint4_t*>(C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j) = v;
       }
-    }
+  } else {
+    const int c_col0 = n0 + wn * S::WN + 4 * fg;
+#pragma unroll
+    for (int i = 0; i < S::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < S::TN; ++j)
+        *reinterpret_cast<float4_t*>(C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j) = acc[i][j];
+  }
 }
+
+#ifndef TFK_GEMM_R64_WAVES_N
+#define TFK_GEMM_R64_WAVES_N 2
+#endif
 
 template <typename OutT>
 int launch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
-  using S = Ring64Shape;
-  auto kern = gemm_ring64_kernel<OutT>;
+  using S = Ring64Shape<TFK_GEMM_R64_WAVES_N>;
+  auto kern = gemm_ring64_kernel<S, OutT>;
   constexpr int lds = S::kUnits * S::kUnitBytes;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
   static thread_local int configured_dev = -1;
