@@ -354,16 +354,31 @@ struct Ring64Shape {
   }
 };
 
-#ifndef TFK_R64_PLAIN_MFMA
-#define TFK_R64_ASM_MFMA
-#endif
 #ifndef TFK_R64_RD_POS
 #define TFK_R64_RD_POS 1
+#endif
+#ifndef TFK_R64_PREP_SLOT
+#define TFK_R64_PREP_SLOT 6
+#endif
+#ifndef TFK_R64_READ_SLOTS
+#define TFK_R64_READ_SLOTS 6
 #endif
 #if defined(TFK_R64_NOREQ)   // timing experiments only: results are wrong without the requests
 #define TFK_R64_REQUEST(...)
 #else
 #define TFK_R64_REQUEST(...) request(__VA_ARGS__)
+#endif
+
+#ifdef TFK_R64_TIMING
+__device__ unsigned long long g_r64_times[4096 * 4];
+#define TFK_R64_STAMP(k)                                                        \
+  do {                                                                          \
+    unsigned long long ts_;                                                     \
+    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ts_)::"memory"); \
+    if (lane == 0) g_r64_times[(blockIdx.x * S::kWaves + wave) * 4 + (k)] = ts_; \
+  } while (0)
+#else
+#define TFK_R64_STAMP(k)
 #endif
 
 template <typename S, typename OutT>
@@ -378,19 +393,22 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * S::BM, n0 = tile_n * S::BN;
   const int wm = wave / S::WAVES_N, wn = wave % S::WAVES_N;
+  TFK_R64_STAMP(0);
 
-  // global -> LDS plan: request n of a wavefront covers rows (wave + kWaves*n) * 8 .. +7 of a
-  // unit; lane l fills physical chunk l % 8 of row l / 8 and fetches the logical chunk the
+  // global -> LDS plan: request n of a wavefront covers rows (wave * kLoads + n) * 8 .. +7 of a
+  // unit (consecutive 1 KiB blocks of LDS, so four requests share one M0 base and differ in the
+  // instruction's immediate offset); lane l fills physical chunk l % 8 of row l / 8 and fetches the logical chunk the
   // swizzle maps there.  A and B share the per-lane offsets (same row stride K); the address
   // is a scalar base (tile origin + k offset) plus this 32-bit per-lane offset, so a request
   // needs no vector arithmetic.
-  const int ld_row = wave * 8 + lane / 8, ld_c = lane % 8;
+  const int ld_row = wave * 8 * S::kLoads + lane / 8, ld_c = lane % 8;
   const char* a_tile = reinterpret_cast<const char*>(A + (size_t)m0 * K);
   const char* b_tile = reinterpret_cast<const char*>(B + (size_t)n0 * K);
   unsigned g_off[S::kLoads];
 #pragma unroll
   for (int n = 0; n < S::kLoads; ++n)
-    g_off[n] = (unsigned)(ld_row + 8 * S::kWaves * n) * (unsigned)K * 2u + (unsigned)S::swizzle(ld_row, ld_c) * 16u;
+    g_off[n] = (unsigned)(ld_row + 8 * n) * (unsigned)K * 2u + (unsigned)S::swizzle(ld_row + 8 * n, ld_c) * 16u -
+               1024u * (n % 4);   // the instruction's immediate offset (added to both addresses) gives it back
   // LDS -> fragment plan: fragment i of k-step ks: row 16*i + l%16 of the wavefront's rows,
   // logical chunk 4*ks + l/16
   const int fr = lane & 15, fg = lane >> 4;
@@ -409,125 +427,69 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
 
   const int num_k_tiles = K / S::BK;
   const unsigned smem_addr = lds_address(smem);
-  // Slot i of a k-step multiplies A fragment i with all B fragments: B needs two full sets,
-  // A fragment i is dead once slot i has issued and is replaced in place by the next k-step's.
-  half8_t af[S::TM], bf[2][S::TN];
+  // Slot i of a k-step multiplies A fragment i with all B fragments; both operands have two
+  // register sets (this k-step's and the next one's).
+  half8_t afx[2][S::TM], bf[2][S::TN];
   // The requests are issued from inline assembly: the compiler then keeps exact counts for the
   // fragment reads (a direct-to-LDS load it knows about makes every LDS wait a full drain),
   // and the vector-memory waits are placed by hand below.
-#ifdef TFK_R64_BUFFER
-  typedef int rsrc_t __attribute__((ext_vector_type(4)));
-  auto make_rsrc = [](const char* base) __attribute__((always_inline)) {
-    const unsigned long long a = (unsigned long long)base;
-    rsrc_t r;
-    r[0] = __builtin_amdgcn_readfirstlane((int)(a & 0xffffffffu));
-    r[1] = __builtin_amdgcn_readfirstlane((int)(a >> 32));
-    r[2] = (int)0xffffffffu;
-    r[3] = 0x00020000;
-    return r;
+  // src: tile origin + k offset (scalar); lds_unit: LDS byte address of this wavefront's first
+  // 1 KiB block in the destination unit.
+  auto request = [&](const char* src, unsigned lds_unit, int n) __attribute__((always_inline)) {
+    if (n % 4 == 0)
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(g_off[n]), "s"(src), "s"(lds_unit + n * 1024)
+                   : "memory");
+    else
+      asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(g_off[n]), "s"(src), "n"(1024 * (n % 4)) : "memory");
   };
-  const rsrc_t a_rsrc = make_rsrc(a_tile), b_rsrc = make_rsrc(b_tile);
-  auto request = [&](const char* tile, int slot, int t, int n) __attribute__((always_inline)) {
-    const unsigned kbyte = (unsigned)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
-    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
-                 :
-                 : "v"(g_off[n]), "s"(tile == a_tile ? a_rsrc : b_rsrc), "s"(kbyte),
-                   "s"(smem_addr + slot * S::kUnitBytes + (wave + S::kWaves * n) * 1024)
-                 : "memory");
-  };
-#else
-  auto request = [&](const char* tile, int slot, int t, int n) __attribute__((always_inline)) {
-    const size_t kbyte = (size_t)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(g_off[n]), "s"(tile + kbyte),
-                   "s"(smem_addr + slot * S::kUnitBytes + (wave + S::kWaves * n) * 1024)
-                 : "memory");
-  };
+  auto k_src = [&](const char* tile, int t) __attribute__((always_inline)) {
+#if defined(TFK_R64_REQ_K0)   // timing experiment only
+    t = min(t, 1);
 #endif
-  // Fragment requests of slot i for the NEXT k-step: the B fragments in the first slots (two
-  // per slot at TN = 8, one at TN = 4; all of them are needed by the next k-step's slot 0),
-  // then its own A fragment.
-  constexpr int kBPerSlot = S::TN / 4;
-  auto frag_part = [&](int slot_a, int slot_b, int ks, int nbuf, int i) __attribute__((always_inline)) {
-    const char* ua = smem + slot_a * S::kUnitBytes;
-    const char* ub = smem + slot_b * S::kUnitBytes;
-    if (i < 4) {
-#pragma unroll
-      for (int f = kBPerSlot * i; f < kBPerSlot * (i + 1); ++f)
-        bf[nbuf][f] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks] + f * 16 * S::kRowBytes);
-    }
-    af[i] = *reinterpret_cast<const half8_t*>(ua + a_rd[ks] + i * 16 * S::kRowBytes);
+    return tile + (size_t)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
   };
-  auto mfma_slot = [&](int buf, int i) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma_16x16x32(bf[buf][j], af[i], acc[i][j]);
-  };
-  // Issue order inside a slot: the fragment reads go between the MFMAs, one at a time (a
-  // 16-cycle MFMA leaves room for one LDS instruction behind it; a cluster of reads stalls the
-  // matrix pipe).  The request sits at the slot boundary.
-  auto interleave = [&](int i) __attribute__((always_inline)) {
-    if constexpr (S::TN == 8) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      if (i < 4) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      } else {
-        __builtin_amdgcn_sched_group_barrier(0x008, 3, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-      }
-    } else {
-      if (i < 4) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      } else {
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-      }
-    }
-  };
-#ifdef TFK_R64_ASM_MFMA
+  const unsigned lds_wave = smem_addr + wave * S::kLoads * 1024;
   // Slot with the MFMAs issued from inline assembly, accumulators pinned to AGPRs, and the
-  // slot's fragment reads placed by hand between them.
-  half8_t afx[2][S::TM];
-  auto slot_pinned = [&](int buf, int i, int slot_a, int slot_b, int ks_next) __attribute__((always_inline)) {
-    const char* ua = smem + slot_a * S::kUnitBytes;
-    const char* ub = smem + slot_b * S::kUnitBytes;
-    constexpr int kReadsB = S::TN / 4;            // B fragments fetched by slots 0..3
-    const int n_reads = (i < 4 ? kReadsB : 0) + 1;
+  // slot's fragment reads placed by hand between them.  (With compiler-issued MFMAs the
+  // register allocator, at exactly 256 live accumulators, shuffles accumulators through VGPRs
+  // whenever the schedule changes slightly.)
+  auto lds_read_b128 = [](unsigned addr) __attribute__((always_inline)) {
+    return *(__attribute__((address_space(3))) const half8_t*)(size_t)addr;
+  };
+  // rd_a / rd_b: this lane's LDS byte address of fragment 0 of the next k-step's A / B operand
+  // (unit base + row + swizzled chunk); fragment f is f * 2 KiB further, in the offset field.
+  auto slot_pinned = [&](int buf, int i, unsigned rd_a, unsigned rd_b) __attribute__((always_inline)) {
+    // The TN + TM fragment reads of the next k-step, B fragments first, are dealt to the first
+    // kReadSlots slots; the last slots read nothing, so the drain in front of the barrier
+    // (and the one at the head of the next k-step) finds the reads already returned.
+    constexpr int kReads = S::TN + S::TM;
+    constexpr int kReadSlots = TFK_R64_READ_SLOTS;
+    const int first = i < kReadSlots ? (i * kReads) / kReadSlots : kReads;
+    const int last = i < kReadSlots ? ((i + 1) * kReads) / kReadSlots : kReads;
+    const int n_reads = last - first;
     int done = 0;
 #pragma unroll
     for (int j = 0; j < S::TN; ++j) {
       asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bf[buf][j]), "v"(afx[buf][i]));
-      // after MFMA j: issue read number `done` if j hits its position (spread evenly)
+      // after MFMA j: issue the next read if j is its position (reads spread evenly over the slot)
       if (done < n_reads && j == (done * S::TN) / n_reads + TFK_R64_RD_POS) {
+        const int q = first + done;
         __builtin_amdgcn_sched_barrier(0);
-        if (i < 4 && done < kReadsB) {
-          const int f = kReadsB * i + done;
-          bf[buf ^ 1][f] = *reinterpret_cast<const half8_t*>(ub + b_rd[ks_next] + f * 16 * S::kRowBytes);
-        } else {
-          afx[buf ^ 1][i] = *reinterpret_cast<const half8_t*>(ua + a_rd[ks_next] + i * 16 * S::kRowBytes);
-        }
+        if (q < S::TN) bf[buf ^ 1][q] = lds_read_b128(rd_b + q * 16 * S::kRowBytes);
+        else afx[buf ^ 1][q - S::TN] = lds_read_b128(rd_a + (q - S::TN) * 16 * S::kRowBytes);
         __builtin_amdgcn_sched_barrier(0);
         ++done;
       }
     }
   };
-#endif
   // Workgroup barrier that keeps the youngest kLoads requests in flight.  The LDS wait and the
   // barrier are builtins so that the compiler knows every earlier fragment read has returned.
   auto ring_barrier = [&]() __attribute__((always_inline)) {
+#ifndef TFK_R64_NOWAIT   // timing experiment: without the wait the results are wrong
     wait_vmem<S::kLoads>();
+#endif
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -538,54 +500,71 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
 #pragma unroll
   for (int u = 0; u < 4; ++u)
 #pragma unroll
-    for (int n = 0; n < S::kLoads; ++n) request(u % 2 ? b_tile : a_tile, u, u / 2, n);
+    for (int n = 0; n < S::kLoads; ++n)
+      request(k_src(u % 2 ? b_tile : a_tile, u / 2), lds_wave + u * S::kUnitBytes, n);
   wait_vmem<2 * S::kLoads>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-#ifdef TFK_R64_ASM_MFMA
 #pragma unroll
   for (int f = 0; f < S::TN; ++f)
     bf[0][f] = *reinterpret_cast<const half8_t*>(smem + S::kUnitBytes + b_rd[0] + f * 16 * S::kRowBytes);
 #pragma unroll
   for (int i = 0; i < S::TM; ++i)
     afx[0][i] = *reinterpret_cast<const half8_t*>(smem + a_rd[0] + i * 16 * S::kRowBytes);
-#else
-#pragma unroll
-  for (int i = 0; i < S::TM; ++i) frag_part(0, 1, 0, 0, i);
-#endif
+  // drained here, visibly to the compiler, so that the waits it places at the head of the loop
+  // only have to cover the loop's own reads
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+  __builtin_amdgcn_sched_barrier(0);
 
-  int sa = 0;   // ring slot of A of tile t; B of tile t is sa+1, A of t+1 sa+2, ... (mod 5)
+  // Ring bookkeeping.  sa = ring slot of A of tile t; B of tile t is sa+1, A of t+1 sa+2, ...
+  // (mod 5).  Everything an iteration needs - the fragment read bases of both k-steps, the two
+  // request destinations and sources - is computed during the PREVIOUS k-step, in the shadow
+  // of its MFMAs, so that no scalar or address arithmetic sits between the last MFMA of one
+  // k-step and the first of the next.
   auto ring = [](int s) __attribute__((always_inline)) { return s >= S::kUnits ? s - S::kUnits : s; };
+  int sa = 0;
+  unsigned rd_a1 = smem_addr + a_rd[1], rd_b1 = smem_addr + S::kUnitBytes + b_rd[1];   // (t, k-step 1)
+  unsigned req_a = lds_wave + 4 * S::kUnitBytes;                                         // A of t+2
+  const char* src_a = k_src(a_tile, 2);
+  unsigned rd_a0 = 0, rd_b0 = 0, req_b = 0;                                               // set in k-step 0
+  const char* src_b = b_tile;
+  TFK_R64_STAMP(1);
   for (int t = 0; t < num_k_tiles; ++t) {
-    const int sb = ring(sa + 1), sa1 = ring(sa + 2), sb1 = ring(sa + 3), sa2 = ring(sa + 4);
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(a_tile, sa2, t + 2, i / kSlotsPerLoad);
-#ifdef TFK_R64_ASM_MFMA
-      slot_pinned(0, i, sa, sb, 1);
-#else
-      mfma_slot(0, i);
-      frag_part(sa, sb, 1, 1, i);
-      interleave(i);
-#endif
+      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(src_a, req_a, i / kSlotsPerLoad);
+      slot_pinned(0, i, rd_a1, rd_b1);
+      if (i == TFK_R64_PREP_SLOT) {   // for k-step 1: reads of (t+1, 0), request of B of t+2 into A of t's slot
+        int s0 = sa, t0 = t;
+        asm volatile("" : "+s"(s0), "+s"(t0));   // keeps the arithmetic below in this slot
+        const int sa1 = ring(s0 + 2), sb1 = ring(s0 + 3);
+        rd_a0 = smem_addr + sa1 * S::kUnitBytes + a_rd[0];
+        rd_b0 = smem_addr + sb1 * S::kUnitBytes + b_rd[0];
+        req_b = lds_wave + s0 * S::kUnitBytes;
+        src_b = k_src(b_tile, t0 + 2);
+        asm volatile("" : "+v"(rd_a0), "+v"(rd_b0), "+s"(req_b), "+s"(src_b));   // ... and not later either
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
     ring_barrier();
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(b_tile, sa, t + 2, i / kSlotsPerLoad);
-#ifdef TFK_R64_ASM_MFMA
-      slot_pinned(1, i, sa1, sb1, 0);
-#else
-      mfma_slot(1, i);
-      frag_part(sa1, sb1, 0, 0, i);
-      interleave(i);
-#endif
+      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(src_b, req_b, i / kSlotsPerLoad);
+      slot_pinned(1, i, rd_a0, rd_b0);
+      if (i == TFK_R64_PREP_SLOT) {   // for the next iteration's k-step 0
+        int s0 = sa, t0 = t;
+        asm volatile("" : "+s"(s0), "+s"(t0));
+        sa = ring(s0 + 2);
+        rd_a1 = smem_addr + sa * S::kUnitBytes + a_rd[1];
+        rd_b1 = smem_addr + ring(sa + 1) * S::kUnitBytes + b_rd[1];
+        req_a = lds_wave + ring(sa + 4) * S::kUnitBytes;
+        src_a = k_src(a_tile, t0 + 3);
+        asm volatile("" : "+v"(rd_a1), "+v"(rd_b1), "+s"(req_a), "+s"(src_a), "+s"(sa));
+      }
     }
-    sa = sa1;
-#ifdef TFK_R64_ASM_MFMA
     // The compiler does not know that the accumulators are written by MFMAs (they are issued
     // from assembly), so nothing would keep it from reading the youngest results right behind
     // the loop without the wait states the matrix pipe needs.  The delay therefore sits inside
@@ -595,19 +574,25 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     int t_seen = t;
     asm volatile("" : "+s"(t_seen));
     if (t_seen + 1 == num_k_tiles) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-#endif
   }
   __builtin_amdgcn_sched_barrier(0);
+  TFK_R64_STAMP(2);
   wait_vmem_all();  // the clamped tail requests must not outlive the workgroup's LDS
   // --- epilogue -----------------------------------------------------------------------------
-  // acc[i][j][r] = C[.. + 16*i + l%16][.. + 16*j + 4*(l/16) + r].  For fp16 output the lanes of
-  // 16-lane groups g and g^1 trade halves of a pair of tiles (v_permlane16_swap): group g even
-  // ends up with 8 consecutive columns of tile j, group g odd with 8 of tile j+1, so every lane
-  // stores 16 bytes and four lanes cover 64 contiguous bytes of a row (8-byte stores cost the
-  // address unit four times as many accesses for the same data).
-  const int c_row0 = m0 + wm * S::WM + fr;
+  // acc[i][j][r] = C[.. + 16*i + l%16][.. + 16*j + 4*(l/16) + r].  For fp16 output the data is
+  // re-dealt so that a store instruction writes 16 rows x 64 contiguous bytes with FOUR
+  // ADJACENT lanes per row: the address unit merges adjacent lanes into one 64-byte access,
+  // whereas lanes 16 apart cost one access each (measured: 64 accesses per instruction and
+  // 9 k cycles of epilogue per wavefront).  Step 1: the 16-lane groups g and g^1 trade halves
+  // of a pair of tiles (v_permlane16_swap), after which group 0/2 holds columns 0-7 / 8-15 of
+  // tile j and group 1/3 the same of tile j+1, 16 bytes per lane.  Step 2: ds_bpermute moves
+  // the 16 bytes of (row r, segment s) to lane 4*r + s.
+  const int c_row0 = m0 + wm * S::WM;
   if constexpr (sizeof(OutT) == 2) {
-    const int c_col0 = n0 + wn * S::WN + 16 * (fg & 1) + 4 * (fg & 2);
+    const int st_row = lane >> 2, st_seg = lane & 3;
+    // segment s of a row lives in group {0, 2, 1, 3}[s] after step 1
+    const int src_lane = st_row + 16 * (((st_seg & 1) << 1) | (st_seg >> 1));
+    OutT* c_lane = C + (size_t)(c_row0 + st_row) * N + n0 + wn * S::WN + 8 * st_seg;
 #pragma unroll
     for (int i = 0; i < S::TM; ++i)
 #pragma unroll
@@ -621,15 +606,18 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
           x[d] = __builtin_bit_cast(unsigned, hx);
           y[d] = __builtin_bit_cast(unsigned, hy);
 #if defined(__HIP_DEVICE_COMPILE__)
-          // odd groups receive x of the group below into x; even groups receive y ... see above:
-          // swap(x, y): x of odd groups <-> y of even groups
+          // x of the odd groups <-> y of the even groups
           auto sw = __builtin_amdgcn_permlane16_swap(x[d], y[d], false, false);
           x[d] = sw[0];
           y[d] = sw[1];
 #endif
         }
-        uint4_t v = {x[0], x[1], y[0], y[1]};
-        *reinterpret_cast<uint4_t*>(C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j) = v;
+        uint4_t v;
+        v[0] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)x[0]);
+        v[1] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)x[1]);
+        v[2] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)y[0]);
+        v[3] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)y[1]);
+        *reinterpret_cast<uint4_t*>(c_lane + (size_t)(16 * i) * N + 16 * j) = v;
       }
   } else {
     const int c_col0 = n0 + wn * S::WN + 4 * fg;
@@ -637,8 +625,12 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     for (int i = 0; i < S::TM; ++i)
 #pragma unroll
       for (int j = 0; j < S::TN; ++j)
-        *reinterpret_cast<float4_t*>(C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j) = acc[i][j];
+        *reinterpret_cast<float4_t*>(C + (size_t)(c_row0 + fr + 16 * i) * N + c_col0 + 16 * j) = acc[i][j];
   }
+#ifdef TFK_R64_TIMING
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  TFK_R64_STAMP(3);
+#endif
 }
 
 #ifndef TFK_GEMM_R64_WAVES_N
@@ -793,6 +785,12 @@ int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStre
 
 }  // namespace
 }  // namespace tfk
+
+#ifdef TFK_R64_TIMING
+extern "C" __attribute__((visibility("default"))) int tf_dbg_r64_times(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tfk::g_r64_times), sizeof(unsigned long long) * n);
+}
+#endif
 
 extern "C" int tf_gemm_f16(const void* A, const void* B, void* C, int c_is_f16, int64_t M,
                            int64_t N, int64_t K, int tm, int tn, int tk, int num_stages,
