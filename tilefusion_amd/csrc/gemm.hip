@@ -7,9 +7,13 @@
 //   * 64-lane wavefronts, v_mfma_f32_16x16x32_f16 base tiles, accumulators in the unified
 //     512-entry register file (one wavefront per SIMD, 128x128 per wavefront at the big tile);
 //   * both operands are K-contiguous, so an MFMA operand fragment is one 16-byte LDS read;
-//   * tiles go global -> LDS without passing through VGPRs (global_load_lds_dwordx4) into a
-//     four-stage, XOR-swizzled LDS ring: a wavefront instruction always writes 1 KiB
-//     of consecutive LDS, so the swizzle is applied on the global (source) side;
+//   * tiles go global -> LDS without passing through VGPRs (global_load_lds_dwordx4) into an
+//     XOR-swizzled LDS ring: a wavefront instruction always writes 1 KiB of consecutive LDS,
+//     so the swizzle is applied on the global (source) side;
+//   * the main kernel (gemm_ring64_kernel) uses 64-deep k-tiles so that every request fetches
+//     whole 128-byte lines, keeps the ring in units of one operand, and issues its MFMAs from
+//     assembly with a hand-placed instruction order (a lone wavefront issues one instruction
+//     per 4 cycles: at most three others fit behind a 16-cycle MFMA);
 //   * workgroup -> tile map keeps the workgroups of one XCD (one L2) on a compact block of
 //     output tiles.
 #include <type_traits>
@@ -327,7 +331,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
 //             (vmcnt leaves only the 8 requests of k-step 0 outstanding);
 //   k-step 1: multiplies (t, 1), reads fragments (t+1, 0), requests B of tile t+2 into the
 //             slot A of tile t left.
-// Every request has at least 8 MFMA slots (1024 MFMA cycles) to land, as in the 4-stage ring.
+// Every request has at least 8 MFMA slots (1024 MFMA cycles) to land.
 // ------------------------------------------------------------------------------------------
 template <int WAVES_N_>
 struct Ring64Shape {
@@ -343,43 +347,8 @@ struct Ring64Shape {
   static_assert(TM == 8 && (TN == 8 || TN == 4) && TM % kLoads == 0, "slot schedule assumes 8 slots per k-step");
   // 128-byte rows: two rows per pass over the banks; chunk ^ (row / 2) % 8 keeps every
   // ds_read_b128 lane pass on 16 different bank groups
-#ifndef TFK_R64_SWZ
-#define TFK_R64_SWZ 0
-#endif
-  __host__ __device__ static constexpr int swizzle(int row, int c) {
-    if (TFK_R64_SWZ == 1) return c ^ (((row / 2) % 4) << 1);   // 32-byte pairs stay in order
-    if (TFK_R64_SWZ == 2) return c ^ (((row / 2) % 2) << 2);   // 64-byte halves stay in order
-    if (TFK_R64_SWZ == 3) return c;
-    return c ^ ((row / 2) % 8);
-  }
+  __host__ __device__ static constexpr int swizzle(int row, int c) { return c ^ ((row / 2) % 8); }
 };
-
-#ifndef TFK_R64_RD_POS
-#define TFK_R64_RD_POS 1
-#endif
-#ifndef TFK_R64_PREP_SLOT
-#define TFK_R64_PREP_SLOT 6
-#endif
-#ifndef TFK_R64_READ_SLOTS
-#define TFK_R64_READ_SLOTS 6
-#endif
-#if defined(TFK_R64_NOREQ)   // timing experiments only: results are wrong without the requests
-#define TFK_R64_REQUEST(...)
-#else
-#define TFK_R64_REQUEST(...) request(__VA_ARGS__)
-#endif
-
-#ifdef TFK_R64_TIMING
-__device__ unsigned long long g_r64_times[4096 * 4];
-#define TFK_R64_STAMP(k)                                                        \
-  do {                                                                          \
-    unsigned long long ts_;                                                     \
-    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(ts_)::"memory"); \
-    if (lane == 0) g_r64_times[(blockIdx.x * S::kWaves + wave) * 4 + (k)] = ts_; \
-  } while (0)
-#else
-#define TFK_R64_STAMP(k)
-#endif
 
 template <typename S, typename OutT>
 __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
@@ -393,7 +362,6 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   tile_of_block(blockIdx.x, gridDim.x, tiles_m, tiles_n, tile_m, tile_n);
   const int m0 = tile_m * S::BM, n0 = tile_n * S::BN;
   const int wm = wave / S::WAVES_N, wn = wave % S::WAVES_N;
-  TFK_R64_STAMP(0);
 
   // global -> LDS plan: request n of a wavefront covers rows (wave * kLoads + n) * 8 .. +7 of a
   // unit (consecutive 1 KiB blocks of LDS, so four requests share one M0 base and differ in the
@@ -445,9 +413,6 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
       asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(g_off[n]), "s"(src), "n"(1024 * (n % 4)) : "memory");
   };
   auto k_src = [&](const char* tile, int t) __attribute__((always_inline)) {
-#if defined(TFK_R64_REQ_K0)   // timing experiment only
-    t = min(t, 1);
-#endif
     return tile + (size_t)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
   };
   const unsigned lds_wave = smem_addr + wave * S::kLoads * 1024;
@@ -460,12 +425,12 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   };
   // rd_a / rd_b: this lane's LDS byte address of fragment 0 of the next k-step's A / B operand
   // (unit base + row + swizzled chunk); fragment f is f * 2 KiB further, in the offset field.
-  auto slot_pinned = [&](int buf, int i, unsigned rd_a, unsigned rd_b) __attribute__((always_inline)) {
+  auto slot_pinned = [&](int buf, int i, unsigned rd_a, unsigned rd_b, auto&& between) __attribute__((always_inline)) {
     // The TN + TM fragment reads of the next k-step, B fragments first, are dealt to the first
     // kReadSlots slots; the last slots read nothing, so the drain in front of the barrier
     // (and the one at the head of the next k-step) finds the reads already returned.
     constexpr int kReads = S::TN + S::TM;
-    constexpr int kReadSlots = TFK_R64_READ_SLOTS;
+    constexpr int kReadSlots = 6;
     const int first = i < kReadSlots ? (i * kReads) / kReadSlots : kReads;
     const int last = i < kReadSlots ? ((i + 1) * kReads) / kReadSlots : kReads;
     const int n_reads = last - first;
@@ -474,22 +439,22 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     for (int j = 0; j < S::TN; ++j) {
       asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bf[buf][j]), "v"(afx[buf][i]));
       // after MFMA j: issue the next read if j is its position (reads spread evenly over the slot)
-      if (done < n_reads && j == (done * S::TN) / n_reads + TFK_R64_RD_POS) {
+      if (done < n_reads && j == (done * S::TN) / n_reads + 1) {
         const int q = first + done;
         __builtin_amdgcn_sched_barrier(0);
         if (q < S::TN) bf[buf ^ 1][q] = lds_read_b128(rd_b + q * 16 * S::kRowBytes);
         else afx[buf ^ 1][q - S::TN] = lds_read_b128(rd_a + (q - S::TN) * 16 * S::kRowBytes);
         __builtin_amdgcn_sched_barrier(0);
         ++done;
+      } else {
+        between(j);   // a piece of scalar bookkeeping, if this gap has one
       }
     }
   };
   // Workgroup barrier that keeps the youngest kLoads requests in flight.  The LDS wait and the
   // barrier are builtins so that the compiler knows every earlier fragment read has returned.
   auto ring_barrier = [&]() __attribute__((always_inline)) {
-#ifndef TFK_R64_NOWAIT   // timing experiment: without the wait the results are wrong
     wait_vmem<S::kLoads>();
-#endif
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -517,53 +482,74 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
   __builtin_amdgcn_sched_barrier(0);
 
-  // Ring bookkeeping.  sa = ring slot of A of tile t; B of tile t is sa+1, A of t+1 sa+2, ...
-  // (mod 5).  Everything an iteration needs - the fragment read bases of both k-steps, the two
-  // request destinations and sources - is computed during the PREVIOUS k-step, in the shadow
-  // of its MFMAs, so that no scalar or address arithmetic sits between the last MFMA of one
-  // k-step and the first of the next.
-  auto ring = [](int s) __attribute__((always_inline)) { return s >= S::kUnits ? s - S::kUnits : s; };
-  int sa = 0;
-  unsigned rd_a1 = smem_addr + a_rd[1], rd_b1 = smem_addr + S::kUnitBytes + b_rd[1];   // (t, k-step 1)
-  unsigned req_a = lds_wave + 4 * S::kUnitBytes;                                         // A of t+2
+  // Ring bookkeeping, in bytes: oa = LDS offset of the unit holding A of tile t; B of tile t is
+  // one unit further, A of t+1 two, ... (mod 5 units).  A wavefront alone on its SIMD issues one
+  // instruction every 4 cycles, so a 16-cycle MFMA hides at most three other instructions:
+  // everything an iteration needs (fragment read bases, request destinations and sources) is
+  // therefore computed during the previous k-step in pieces of at most three instructions,
+  // each pinned into its own gap between two MFMAs of the slots that carry no fragment reads.
+  constexpr unsigned kRingBytes = S::kUnits * S::kUnitBytes;
+  auto ring = [](unsigned o) __attribute__((always_inline)) { return o >= kRingBytes ? o - kRingBytes : o; };
+  const unsigned rdbase_a0 = smem_addr + a_rd[0], rdbase_a1 = smem_addr + a_rd[1];
+  const unsigned rdbase_b0 = smem_addr + b_rd[0], rdbase_b1 = smem_addr + b_rd[1];
+  const int last_tile = num_k_tiles - 1;
+  unsigned oa = 0;                                             // A of tile t
+  unsigned oa1 = 2 * S::kUnitBytes, ob1 = 3 * S::kUnitBytes;   // A, B of tile t+1
+  unsigned rd_a1 = rdbase_a1, rd_b1 = rdbase_b1 + S::kUnitBytes;   // reads of (t, k-step 1)
+  unsigned req_a = lds_wave + 4 * S::kUnitBytes;                   // A of t+2
   const char* src_a = k_src(a_tile, 2);
-  unsigned rd_a0 = 0, rd_b0 = 0, req_b = 0;                                               // set in k-step 0
+  unsigned rd_a0 = 0, rd_b0 = 0, req_b = 0;                        // set during k-step 0
   const char* src_b = b_tile;
-  TFK_R64_STAMP(1);
+  int kt = 0;
+#define TFK_PIN_S(x) asm volatile("" : "+s"(x))
+#define TFK_PIN_V(x) asm volatile("" : "+v"(x))
+  // pieces run in the gaps of slot kPrepSlot (and the one after it) of k-step 0 / k-step 1
+  auto prep0 = [&](int step, int t) __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    switch (step) {
+      case 0: TFK_PIN_S(oa); oa1 = ring(oa + 2 * S::kUnitBytes); TFK_PIN_S(oa1); break;
+      case 1: ob1 = ring(oa1 + S::kUnitBytes); TFK_PIN_S(ob1); break;
+      case 2: rd_a0 = rdbase_a0 + oa1; TFK_PIN_V(rd_a0); break;
+      case 3: rd_b0 = rdbase_b0 + ob1; TFK_PIN_V(rd_b0); break;
+      case 4: req_b = lds_wave + oa; TFK_PIN_S(req_b); break;
+      case 5: kt = t; TFK_PIN_S(kt); kt = min(kt + 2, last_tile); TFK_PIN_S(kt); break;
+      case 6: src_b = b_tile + (size_t)(unsigned)(kt * (S::BK * 2)); TFK_PIN_S(src_b); break;
+      default: break;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto prep1 = [&](int step, int t) __attribute__((always_inline)) {
+    __builtin_amdgcn_sched_barrier(0);
+    switch (step) {
+      case 0: oa = oa1; TFK_PIN_S(oa); rd_a1 = rdbase_a1 + oa; TFK_PIN_V(rd_a1); break;
+      case 1: rd_b1 = rdbase_b1 + ob1; TFK_PIN_V(rd_b1); break;
+      case 2: req_a = ring(oa + 4 * S::kUnitBytes); TFK_PIN_S(req_a); break;
+      case 3: req_a += lds_wave; TFK_PIN_S(req_a); break;
+      case 4: kt = t; TFK_PIN_S(kt); kt = min(kt + 3, last_tile); TFK_PIN_S(kt); break;
+      case 5: src_a = a_tile + (size_t)(unsigned)(kt * (S::BK * 2)); TFK_PIN_S(src_a); break;
+      default: break;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  constexpr int kPrepSlot = 6;   // slots 6 and 7 carry no fragment reads
   for (int t = 0; t < num_k_tiles; ++t) {
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(src_a, req_a, i / kSlotsPerLoad);
-      slot_pinned(0, i, rd_a1, rd_b1);
-      if (i == TFK_R64_PREP_SLOT) {   // for k-step 1: reads of (t+1, 0), request of B of t+2 into A of t's slot
-        int s0 = sa, t0 = t;
-        asm volatile("" : "+s"(s0), "+s"(t0));   // keeps the arithmetic below in this slot
-        const int sa1 = ring(s0 + 2), sb1 = ring(s0 + 3);
-        rd_a0 = smem_addr + sa1 * S::kUnitBytes + a_rd[0];
-        rd_b0 = smem_addr + sb1 * S::kUnitBytes + b_rd[0];
-        req_b = lds_wave + s0 * S::kUnitBytes;
-        src_b = k_src(b_tile, t0 + 2);
-        asm volatile("" : "+v"(rd_a0), "+v"(rd_b0), "+s"(req_b), "+s"(src_b));   // ... and not later either
-      }
+      if (i % kSlotsPerLoad == 0) request(src_a, req_a, i / kSlotsPerLoad);
+      slot_pinned(0, i, rd_a1, rd_b1, [&](int j) __attribute__((always_inline)) {
+        if (i >= kPrepSlot) prep0((i - kPrepSlot) * S::TN + j, t);
+      });
     }
     __builtin_amdgcn_sched_barrier(0);
     ring_barrier();
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) TFK_R64_REQUEST(src_b, req_b, i / kSlotsPerLoad);
-      slot_pinned(1, i, rd_a0, rd_b0);
-      if (i == TFK_R64_PREP_SLOT) {   // for the next iteration's k-step 0
-        int s0 = sa, t0 = t;
-        asm volatile("" : "+s"(s0), "+s"(t0));
-        sa = ring(s0 + 2);
-        rd_a1 = smem_addr + sa * S::kUnitBytes + a_rd[1];
-        rd_b1 = smem_addr + ring(sa + 1) * S::kUnitBytes + b_rd[1];
-        req_a = lds_wave + ring(sa + 4) * S::kUnitBytes;
-        src_a = k_src(a_tile, t0 + 3);
-        asm volatile("" : "+v"(rd_a1), "+v"(rd_b1), "+s"(req_a), "+s"(src_a), "+s"(sa));
-      }
+      if (i % kSlotsPerLoad == 0) request(src_b, req_b, i / kSlotsPerLoad);
+      slot_pinned(1, i, rd_a0, rd_b0, [&](int j) __attribute__((always_inline)) {
+        if (i >= kPrepSlot) prep1((i - kPrepSlot) * S::TN + j, t);
+      });
     }
     // The compiler does not know that the accumulators are written by MFMAs (they are issued
     // from assembly), so nothing would keep it from reading the youngest results right behind
@@ -576,7 +562,6 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     if (t_seen + 1 == num_k_tiles) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   }
   __builtin_amdgcn_sched_barrier(0);
-  TFK_R64_STAMP(2);
   wait_vmem_all();  // the clamped tail requests must not outlive the workgroup's LDS
   // --- epilogue -----------------------------------------------------------------------------
   // acc[i][j][r] = C[.. + 16*i + l%16][.. + 16*j + 4*(l/16) + r].  For fp16 output the data is
@@ -627,10 +612,6 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
       for (int j = 0; j < S::TN; ++j)
         *reinterpret_cast<float4_t*>(C + (size_t)(c_row0 + fr + 16 * i) * N + c_col0 + 16 * j) = acc[i][j];
   }
-#ifdef TFK_R64_TIMING
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  TFK_R64_STAMP(3);
-#endif
 }
 
 #ifndef TFK_GEMM_R64_WAVES_N
@@ -785,12 +766,6 @@ int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStre
 
 }  // namespace
 }  // namespace tfk
-
-#ifdef TFK_R64_TIMING
-extern "C" __attribute__((visibility("default"))) int tf_dbg_r64_times(unsigned long long* host, int n) {
-  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(tfk::g_r64_times), sizeof(unsigned long long) * n);
-}
-#endif
 
 extern "C" int tf_gemm_f16(const void* A, const void* B, void* C, int c_is_f16, int64_t M,
                            int64_t N, int64_t K, int tm, int tn, int tk, int num_stages,
