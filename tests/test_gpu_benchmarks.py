@@ -1,0 +1,30 @@
+"""The micro-benchmarks under benchmarks/ run on the GPU and check their own results."""
+
+import io
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_g2s_copy_benchmark_checks_itself():
+    d = os.path.join(ROOT, "benchmarks", "cpp", "g2s_copy")
+    path = os.path.join(d, "g2s_copy")
+    if not os.path.exists(path):
+        subprocess.check_call(["make", "-C", d])
+    out = subprocess.run([path], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert out.stdout.count("|ok|") == 11 and "all configurations ok" in out.stdout
+
+
+def test_fused_two_gemms_sweep_is_correct_on_a_few_shapes():
+    sys.path.insert(0, os.path.join(ROOT, "benchmarks", "fused_two_gemms"))
+    import bench as fused_bench
+
+    buf = io.StringIO()
+    assert fused_bench.run(shapes=[(512, 512), (2048, 2048), (4096, 1024)], out=buf), buf.getvalue()
+    assert "MISMATCH" not in buf.getvalue()

@@ -403,14 +403,13 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   // and the vector-memory waits are placed by hand below.
   // src: tile origin + k offset (scalar); lds_unit: LDS byte address of this wavefront's first
   // 1 KiB block in the destination unit.
-  auto request = [&](const char* src, unsigned lds_unit, int n) __attribute__((always_inline)) {
-    if (n % 4 == 0)
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                   :
-                   : "v"(g_off[n]), "s"(src), "s"(lds_unit + n * 1024)
-                   : "memory");
-    else
-      asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(g_off[n]), "s"(src), "n"(1024 * (n % 4)) : "memory");
+  // M0 (the LDS destination of requests n .. n+3, n % 4 == 0) is written one MFMA gap ahead of
+  // the first of them, which saves the wait state an M0 write needs in front of its use.
+  auto set_m0 = [&](unsigned lds_unit, int n) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %0" : : "s"(lds_unit + n * 1024) : "memory");
+  };
+  auto request = [&](const char* src, int n) __attribute__((always_inline)) {
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(g_off[n]), "s"(src), "n"(1024 * (n % 4)) : "memory");
   };
   auto k_src = [&](const char* tile, int t) __attribute__((always_inline)) {
     return tile + (size_t)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
@@ -454,8 +453,8 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   // Workgroup barrier that keeps the youngest kLoads requests in flight.  The LDS wait and the
   // barrier are builtins so that the compiler knows every earlier fragment read has returned.
   auto ring_barrier = [&]() __attribute__((always_inline)) {
-    wait_vmem<S::kLoads>();
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    // one s_waitcnt: vmcnt(kLoads) lgkmcnt(0); a builtin, so the compiler knows the LDS part
+    __builtin_amdgcn_s_waitcnt((S::kLoads & 15) | 0x70 | ((S::kLoads >> 4) << 14));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
@@ -465,8 +464,13 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
 #pragma unroll
   for (int u = 0; u < 4; ++u)
 #pragma unroll
-    for (int n = 0; n < S::kLoads; ++n)
-      request(k_src(u % 2 ? b_tile : a_tile, u / 2), lds_wave + u * S::kUnitBytes, n);
+    for (int n = 0; n < S::kLoads; ++n) {
+      if (n % 4 == 0) {
+        set_m0(lds_wave + u * S::kUnitBytes, n);
+        asm volatile("s_nop 0");
+      }
+      request(k_src(u % 2 ? b_tile : a_tile, u / 2), n);
+    }
   wait_vmem<2 * S::kLoads>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
@@ -532,13 +536,25 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     __builtin_amdgcn_sched_barrier(0);
   };
   constexpr int kPrepSlot = 6;   // slots 6 and 7 carry no fragment reads
+  // request n of a k-step goes at the head of slot n * kSlotsPerLoad; if n % 4 == 0 its M0 is
+  // written in the last gap of the slot before (for slot 0: of the previous k-step's slot 7)
+  auto m0_slot = [&](int i, int j, unsigned next_unit, unsigned this_unit) __attribute__((always_inline)) {
+    if (j != S::TN - 1) return;
+    const int i_next = (i + 1) % S::TM;
+    if (i_next % kSlotsPerLoad != 0 || (i_next / kSlotsPerLoad) % 4 != 0) return;
+    __builtin_amdgcn_sched_barrier(0);
+    set_m0(i_next == 0 ? next_unit : this_unit, i_next / kSlotsPerLoad);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  set_m0(req_a, 0);
   for (int t = 0; t < num_k_tiles; ++t) {
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) request(src_a, req_a, i / kSlotsPerLoad);
+      if (i % kSlotsPerLoad == 0) request(src_a, i / kSlotsPerLoad);
       slot_pinned(0, i, rd_a1, rd_b1, [&](int j) __attribute__((always_inline)) {
         if (i >= kPrepSlot) prep0((i - kPrepSlot) * S::TN + j, t);
+        m0_slot(i, j, req_b, req_a);
       });
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -546,9 +562,10 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) request(src_b, req_b, i / kSlotsPerLoad);
+      if (i % kSlotsPerLoad == 0) request(src_b, i / kSlotsPerLoad);
       slot_pinned(1, i, rd_a0, rd_b0, [&](int j) __attribute__((always_inline)) {
         if (i >= kPrepSlot) prep1((i - kPrepSlot) * S::TN + j, t);
+        m0_slot(i, j, req_a, req_b);
       });
     }
     // The compiler does not know that the accumulators are written by MFMAs (they are issued
