@@ -45,6 +45,68 @@ TFK_DEVICE void tile_to_lds(const half_t* __restrict__ g, size_t ld, char* lds, 
   }
 }
 
+// The two products of one n-tile for one wavefront, with the LDS fragment reads issued one
+// step ahead of the MFMAs that use them (a wavefront alone on its SIMD has nobody to hide the
+// LDS latency behind; requesting step s+1 before multiplying step s takes it off the critical
+// path).  sB: [TN][KC] tile, sC: [TP][TN] tile, both XOR-swizzled.
+//   first_product:  acc1[nt] += S^T tile (rows n from B, columns m from A) over the KC / 32 steps
+//   second_product: acc2[pt] += (fp16 of acc1) * C over the TN / 32 steps; lane (m = lr, group
+//                   lg) holds A*B[m][16*nt + 4*lg + r] in acc1[nt][r], and reduction step s uses
+//                   n = 32*s + {4*lg + 0..3, 16 + 4*lg + 0..3} as its 8 slots.
+template <int TN, int KC>
+TFK_DEVICE void first_product(const char* sB, const half8_t* af, float4_t* acc1, int lr, int lg) {
+  constexpr int kNT = TN / 16, kKSteps = KC / 32, kCh = KC / 8;
+  half8_t bf[2][kNT];
+  auto read_b = [&](int buf, int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) {
+      const int row = nt * 16 + lr;
+      bf[buf][nt] = *reinterpret_cast<const half8_t*>(sB + row * KC * 2 + swz<kCh>(row, ks * 4 + lg) * 16);
+    }
+  };
+  read_b(0, 0);
+#pragma unroll
+  for (int ks = 0; ks < kKSteps; ++ks) {
+    if (ks + 1 < kKSteps) read_b((ks + 1) & 1, ks + 1);
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) acc1[nt] = mfma_16x16x32(bf[ks & 1][nt], af[ks], acc1[nt]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+template <int TN, int TP>
+TFK_DEVICE void second_product(const char* sC, const float4_t* acc1, float4_t* acc2, int lr, int lg) {
+  constexpr int kPT = TP / 16, kSteps = TN / 32, kCh = TN / 8;
+  half8_t cf[2][kPT];
+  auto read_c = [&](int buf, int s2) __attribute__((always_inline)) {
+#pragma unroll
+    for (int pt = 0; pt < kPT; ++pt) {
+      const int row = pt * 16 + lr;
+      const char* base = sC + row * TN * 2 + (lg & 1) * 8;
+      const half4_t lo = *reinterpret_cast<const half4_t*>(base + swz<kCh>(row, 4 * s2 + (lg >> 1)) * 16);
+      const half4_t hi = *reinterpret_cast<const half4_t*>(base + swz<kCh>(row, 4 * s2 + 2 + (lg >> 1)) * 16);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        cf[buf][pt][r] = lo[r];
+        cf[buf][pt][4 + r] = hi[r];
+      }
+    }
+  };
+  read_c(0, 0);
+#pragma unroll
+  for (int s2 = 0; s2 < kSteps; ++s2) {
+    if (s2 + 1 < kSteps) read_c((s2 + 1) & 1, s2 + 1);
+    half8_t pa;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      pa[r] = (half_t)acc1[2 * s2][r];
+      pa[4 + r] = (half_t)acc1[2 * s2 + 1][r];
+    }
+#pragma unroll
+    for (int pt = 0; pt < kPT; ++pt) acc2[pt] = mfma_16x16x32(pa, cf[s2 & 1][pt], acc2[pt]);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 template <int TN, int TP, int KC>
 __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
     const half_t* __restrict__ A, const half_t* __restrict__ B, const half_t* __restrict__ C,
@@ -91,43 +153,9 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
         af[ks] = *reinterpret_cast<const half8_t*>(a_ptr + k0 + ks * 32);
       wait_vmem_all();
       __syncthreads();
-#pragma unroll
-      for (int ks = 0; ks < kKSteps; ++ks)
-#pragma unroll
-        for (int nt = 0; nt < kNT; ++nt) {
-          const int row = nt * 16 + lr;
-          const half8_t bf = *reinterpret_cast<const half8_t*>(
-              sB + row * KC * 2 + swz<kBChunks>(row, ks * 4 + lg) * 16);
-          // S^T tile: rows n (from B), columns m (from A)
-          acc1[nt] = mfma_16x16x32(bf, af[ks], acc1[nt]);
-        }
+      first_product<TN, KC>(sB, af, acc1, lr, lg);
     }
-
-    // Second GEMM.  Lane (m = lr, group lg) holds A*B[m][16*nt + 4*lg + r] in acc1[nt][r];
-    // reduction step s uses n = 32*s + {4*lg + 0..3, 16 + 4*lg + 0..3} as its 8 slots.
-#pragma unroll
-    for (int s = 0; s < TN / 32; ++s) {
-      half8_t pa;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        pa[r] = (half_t)acc1[2 * s][r];
-        pa[4 + r] = (half_t)acc1[2 * s + 1][r];
-      }
-#pragma unroll
-      for (int pt = 0; pt < kPT; ++pt) {
-        const int row = pt * 16 + lr;
-        const char* base = sC + row * TN * 2 + (lg & 1) * 8;
-        const half4_t lo = *reinterpret_cast<const half4_t*>(base + swz<kCChunks>(row, 4 * s + (lg >> 1)) * 16);
-        const half4_t hi = *reinterpret_cast<const half4_t*>(base + swz<kCChunks>(row, 4 * s + 2 + (lg >> 1)) * 16);
-        half8_t cf;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          cf[r] = lo[r];
-          cf[4 + r] = hi[r];
-        }
-        acc2[pt] = mfma_16x16x32(pa, cf, acc2[pt]);
-      }
-    }
+    second_product<TN, TP>(sC, acc1, acc2, lr, lg);
   }
 
   // Epilogue: acc2[pt][r] = D[m0 + 16*wave + 4*lg + r][p0 + 16*pt + lr]
@@ -257,38 +285,8 @@ __global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
     float4_t acc1[TN / 16];
 #pragma unroll
     for (int nt = 0; nt < TN / 16; ++nt) acc1[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-      for (int nt = 0; nt < TN / 16; ++nt) {
-        const int row = nt * 16 + lr;
-        const half8_t bf = *reinterpret_cast<const half8_t*>(sB + row * K * 2 + swz<16>(row, ks * 4 + lg) * 16);
-        acc1[nt] = mfma_16x16x32(bf, af[ks], acc1[nt]);   // S^T tile: rows n, columns m
-      }
-    // second product: see fused_two_gemms_kernel for the layout argument
-#pragma unroll
-    for (int s2 = 0; s2 < TN / 32; ++s2) {
-      half8_t pa;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        pa[r] = (half_t)acc1[2 * s2][r];
-        pa[4 + r] = (half_t)acc1[2 * s2 + 1][r];
-      }
-#pragma unroll
-      for (int pt = 0; pt < 8; ++pt) {
-        const int row = pt * 16 + lr;
-        const char* base = sC + row * TN * 2 + (lg & 1) * 8;
-        const half4_t lo = *reinterpret_cast<const half4_t*>(base + swz<8>(row, 4 * s2 + (lg >> 1)) * 16);
-        const half4_t hi = *reinterpret_cast<const half4_t*>(base + swz<8>(row, 4 * s2 + 2 + (lg >> 1)) * 16);
-        half8_t cf;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          cf[r] = lo[r];
-          cf[4 + r] = hi[r];
-        }
-        acc2[pt] = mfma_16x16x32(pa, cf, acc2[pt]);
-      }
-    }
+    first_product<TN, K>(sB, af, acc1, lr, lg);
+    second_product<TN, P>(sC, acc1, acc2, lr, lg);
   }
   wait_vmem_all();  // the surplus requests must not outlive the workgroup's LDS
 
