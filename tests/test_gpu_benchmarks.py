@@ -22,9 +22,24 @@ def test_g2s_copy_benchmark_checks_itself():
 
 
 def test_fused_two_gemms_sweep_is_correct_on_a_few_shapes():
-    sys.path.insert(0, os.path.join(ROOT, "benchmarks", "fused_two_gemms"))
-    import bench as fused_bench
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("fused_bench", os.path.join(ROOT, "benchmarks", "fused_two_gemms", "bench.py"))
+    fused_bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(fused_bench)
 
     buf = io.StringIO()
     assert fused_bench.run(shapes=[(512, 512), (2048, 2048), (4096, 1024)], out=buf), buf.getvalue()
+    assert "MISMATCH" not in buf.getvalue()
+
+
+def test_gemm_sweep_is_correct_on_the_small_shapes():
+    sys.path.insert(0, os.path.join(ROOT, "benchmarks", "gemm"))
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("gemm_bench", os.path.join(ROOT, "benchmarks", "gemm", "bench.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    buf = io.StringIO()
+    assert mod.run(shapes=mod.SHAPES[:5], out=buf), buf.getvalue()
     assert "MISMATCH" not in buf.getvalue()
