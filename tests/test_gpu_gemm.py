@@ -69,12 +69,13 @@ def test_integer_inputs_are_exact():
         assert torch.equal(c.float().cpu(), N.gemm_ref(a, b))
 
 
-# The 256x256x64 ring kernel (>= 128 tiles of 256x256, K % 64 == 0): one k-tile, fewer k-tiles
-# than ring units, counts that are not multiples of the ring length, non-square tile grids.
+# The 256x256x64 ring kernel (grids of more than 128 tiles of 256x256, K % 64 == 0): one k-tile,
+# fewer k-tiles than ring units, counts that are not multiples of the ring length, non-square
+# tile grids.
 # Small integers make every product and partial sum exact, so the comparison is bit-exact and
 # a single misplaced fragment, a stale ring unit or a missed wait cannot hide in a tolerance.
-@pytest.mark.parametrize("m,n,k", [(4096, 2048, 64), (2048, 4096, 128), (4096, 4096, 192), (2048, 4096, 320),
-                                   (8192, 1024, 448), (4096, 4096, 1088)])
+@pytest.mark.parametrize("m,n,k", [(4096, 3072, 64), (3072, 4096, 128), (4096, 4096, 192), (2304, 4096, 320),
+                                   (6144, 2048, 448), (4096, 4096, 1088)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
 def test_ring_kernel_exact(m, n, k, out_dtype):
     g = torch.Generator(device=DEV).manual_seed(m + 3 * n + 7 * k)
@@ -88,6 +89,25 @@ def test_ring_kernel_exact(m, n, k, out_dtype):
     # and against the CPU oracle on a sampled block (the oracle is the reference, torch only scales it up)
     blk = N.gemm_ref(a[256:384].cpu(), b[512:576].cpu())
     assert torch.equal(c[256:384, 512:576].float().cpu(), blk if out_dtype == torch.float32 else blk.half().float())
+
+
+# The same ring kernel with 128x128 tiles (grids with fewer than 128 tiles of 256x256; a ring of
+# 9 units, requests 4 tiles ahead): fewer k-tiles than the look-ahead, counts around the ring
+# length, one tile, non-square grids.
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (128, 256, 128), (256, 128, 256), (384, 640, 320), (640, 384, 576),
+                                   (1024, 1024, 1216), (2048, 2048, 2048)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_ring_kernel_mid_tiles_exact(m, n, k, out_dtype):
+    g = torch.Generator(device=DEV).manual_seed(m + 3 * n + 7 * k)
+    a = torch.randint(-2, 3, (m, k), generator=g, device=DEV).half()
+    b = torch.randint(-2, 3, (n, k), generator=g, device=DEV).half()
+    c = c_gemm(a, b, out_dtype)
+    ref = torch.matmul(a.float(), b.float().T)
+    if out_dtype == torch.float16:
+        ref = ref.half()   # |values| <= 4k = 8192 at most; sums of a few thousand terms of size <= 4 stay far below it
+    assert torch.equal(c, ref)
+    blk = N.gemm_ref(a[:128].cpu(), b[64:128].cpu())
+    assert torch.equal(c[:128, 64:128].float().cpu(), blk if out_dtype == torch.float32 else blk.half().float())
 
 
 def test_linearity_at_full_size():

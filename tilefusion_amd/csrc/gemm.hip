@@ -13,7 +13,10 @@
 //   * the main kernel (gemm_ring64_kernel) uses 64-deep k-tiles so that every request fetches
 //     whole 128-byte lines, keeps the ring in units of one operand, and issues its MFMAs from
 //     assembly with a hand-placed instruction order (a lone wavefront issues one instruction
-//     per 4 cycles: at most three others fit behind a 16-cycle MFMA);
+//     per 4 cycles: at most three others fit behind a 16-cycle MFMA); it comes with 256 x 256
+//     tiles and, for grids that those would leave most CUs idle on, with 128 x 128 tiles;
+//     K % 64 != 0 falls back to the 32-deep direct-to-LDS kernel, other shapes to a
+//     bounds-checked one;
 //   * workgroup -> tile map keeps the workgroups of one XCD (one L2) on a compact block of
 //     output tiles.
 #include <type_traits>
@@ -333,18 +336,74 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
 //             slot A of tile t left.
 // Every request has at least 8 MFMA slots (1024 MFMA cycles) to land.
 // ------------------------------------------------------------------------------------------
-template <int WAVES_N_>
+//
+// The same kernel serves 128 x 128 tiles (2 x 2 wavefronts of 64 x 64, units of 16 KiB) for
+// grids that 256 x 256 tiles would leave most CUs idle on.  Its k-steps are four times
+// shorter, so requests run kAhead = 4 tiles ahead (a ring of 2 * kAhead + 1 = 9 units).
+template <int BM_, int WAVES_N_, int AHEAD_>
 struct Ring64Shape {
-  static constexpr int BM = 256, BN = 256, BK = 64;
+  static constexpr int BM = BM_, BN = BM_, BK = 64;
   static constexpr int WAVES_M = 2, WAVES_N = WAVES_N_;
   static constexpr int kWaves = WAVES_M * WAVES_N, kThreads = kWaves * kWaveSize;
   static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   static constexpr int TM = WM / 16, TN = WN / 16;          // 16x16 MFMA tiles per wavefront
   static constexpr int kRowBytes = BK * 2;                  // 128
-  static constexpr int kUnitBytes = BM * kRowBytes;         // 32 KiB: one operand of one tile
-  static constexpr int kUnits = 5;
+  static constexpr int kUnitBytes = BM * kRowBytes;         // one operand of one tile
+  static constexpr int kAhead = AHEAD_;                     // tiles between a request and its use
+  static constexpr int kUnits = 2 * kAhead + 1;
   static constexpr int kLoads = BM / 8 / kWaves;            // 1 KiB requests per wavefront and unit
-  static_assert(TM == 8 && (TN == 8 || TN == 4) && TM % kLoads == 0, "slot schedule assumes 8 slots per k-step");
+  // slot schedule of a k-step (TM slots of TN MFMAs): the TM + TN fragment reads of the next
+  // k-step are dealt to the first kReadSlots slots; the scalar bookkeeping runs in the gaps
+  // without a read from slot kPrepSlot on
+  static constexpr int kReads = TM + TN;
+  static constexpr int kReadSlots = TM == 8 ? 6 : TM - 1;
+  static constexpr int kPrepSlot = TM == 8 ? 6 : 0;
+  static constexpr int reads_first(int i) { return i < kReadSlots ? (i * kReads) / kReadSlots : kReads; }
+  static constexpr int reads_in(int i) { return reads_first(i + 1) - reads_first(i); }
+  // read number d of a slot follows MFMA (d * TN) / n of that slot (gap j = that + 1)
+  static constexpr bool gap_has_read(int i, int j) {
+    const int n = reads_in(i);
+    for (int d = 0; d < n; ++d)
+      if (j == (d * TN) / n + 1) return true;
+    return false;
+  }
+  // which bookkeeping piece runs in gap j of slot i (-1: none); a table, so that the unrolled
+  // slots index it with constants
+  struct PrepTable {
+    int piece[TM * TN];
+  };
+  static constexpr PrepTable make_prep_table() {
+    PrepTable t{};
+    int rank = 0;
+    for (int i = 0; i < TM; ++i)
+      for (int j = 0; j < TN; ++j) t.piece[i * TN + j] = (i < kPrepSlot || gap_has_read(i, j)) ? -1 : rank++;
+    return t;
+  }
+  static constexpr PrepTable kPrep = make_prep_table();
+  static constexpr int free_gaps() { return kPrep.piece[TM * TN - 1] + 1; }
+  static constexpr bool reads_fit() {
+    for (int i = 0; i < TM; ++i) {
+      if (reads_in(i) > TN - 1) return false;
+      for (int d = 1; d < reads_in(i); ++d)   // two reads never share a gap
+        if ((d * TN) / reads_in(i) == ((d - 1) * TN) / reads_in(i)) return false;
+    }
+    return true;
+  }
+  static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4) && TM % kLoads == 0 && kLoads % 4 == 0,
+                "slot schedule: a request every TM / kLoads slots, M0 shared by four requests");
+  // M0 is written in the last gap of the slot in front of requests 0, 4, ...
+  static constexpr bool m0_slot_after(int i) {
+    const int i_next = (i + 1) % TM;
+    return i_next % (TM / kLoads) == 0 && (i_next / (TM / kLoads)) % 4 == 0;
+  }
+  static constexpr bool m0_gaps_free() {
+    for (int i = 0; i < TM; ++i)
+      if (m0_slot_after(i) && gap_has_read(i, TN - 1)) return false;
+    return true;
+  }
+  static_assert(reads_fit() && free_gaps() >= 7 && m0_gaps_free(),
+                "slot schedule: every read, bookkeeping piece and M0 write needs its own gap");
+  static_assert((2 * kAhead - 3) * kLoads < 64, "vmcnt is a 6-bit counter");
   // 128-byte rows: two rows per pass over the banks; chunk ^ (row / 2) % 8 keeps every
   // ds_read_b128 lane pass on 16 different bank groups
   __host__ __device__ static constexpr int swizzle(int row, int c) { return c ^ ((row / 2) % 8); }
@@ -426,13 +485,10 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   // (unit base + row + swizzled chunk); fragment f is f * 2 KiB further, in the offset field.
   auto slot_pinned = [&](int buf, int i, unsigned rd_a, unsigned rd_b, auto&& between) __attribute__((always_inline)) {
     // The TN + TM fragment reads of the next k-step, B fragments first, are dealt to the first
-    // kReadSlots slots; the last slots read nothing, so the drain in front of the barrier
+    // kReadSlots slots; the last slot(s) read nothing, so the drain in front of the barrier
     // (and the one at the head of the next k-step) finds the reads already returned.
-    constexpr int kReads = S::TN + S::TM;
-    constexpr int kReadSlots = 6;
-    const int first = i < kReadSlots ? (i * kReads) / kReadSlots : kReads;
-    const int last = i < kReadSlots ? ((i + 1) * kReads) / kReadSlots : kReads;
-    const int n_reads = last - first;
+    const int first = S::reads_first(i);
+    const int n_reads = S::reads_in(i);
     int done = 0;
 #pragma unroll
     for (int j = 0; j < S::TN; ++j) {
@@ -450,19 +506,22 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
       }
     }
   };
-  // Workgroup barrier that keeps the youngest kLoads requests in flight.  The LDS wait and the
+  // Workgroup barrier in the middle of tile t: tile t+1 must have landed, the requests of
+  // tiles t+2 .. t+kAhead-1 and of this tile's k-step 0 stay in flight.  The LDS wait and the
   // barrier are builtins so that the compiler knows every earlier fragment read has returned.
+  constexpr int kInFlight = (2 * S::kAhead - 3) * S::kLoads;
   auto ring_barrier = [&]() __attribute__((always_inline)) {
-    // one s_waitcnt: vmcnt(kLoads) lgkmcnt(0); a builtin, so the compiler knows the LDS part
-    __builtin_amdgcn_s_waitcnt((S::kLoads & 15) | 0x70 | ((S::kLoads >> 4) << 14));
+    // one s_waitcnt: vmcnt(kInFlight) lgkmcnt(0); a builtin, so the compiler knows the LDS part
+    __builtin_amdgcn_s_waitcnt((kInFlight & 15) | 0x70 | ((kInFlight >> 4) << 14));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
   };
   constexpr int kSlotsPerLoad = S::TM / S::kLoads;   // a request every so many slots
 
-  // prologue: tiles 0 and 1 into ring slots 0..3; fragments (0, 0) once tile 0 is there
+  // prologue: tiles 0 .. kAhead-1 into the first 2 * kAhead units; fragments (0, 0) once
+  // tile 0 is there
 #pragma unroll
-  for (int u = 0; u < 4; ++u)
+  for (int u = 0; u < 2 * S::kAhead; ++u)
 #pragma unroll
     for (int n = 0; n < S::kLoads; ++n) {
       if (n % 4 == 0) {
@@ -471,7 +530,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
       }
       request(k_src(u % 2 ? b_tile : a_tile, u / 2), n);
     }
-  wait_vmem<2 * S::kLoads>();
+  wait_vmem<2 * (S::kAhead - 1) * S::kLoads>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
 #pragma unroll
@@ -487,7 +546,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   __builtin_amdgcn_sched_barrier(0);
 
   // Ring bookkeeping, in bytes: oa = LDS offset of the unit holding A of tile t; B of tile t is
-  // one unit further, A of t+1 two, ... (mod 5 units).  A wavefront alone on its SIMD issues one
+  // one unit further, A of t+1 two, ... (mod kUnits units).  A wavefront alone on its SIMD issues one
   // instruction every 4 cycles, so a 16-cycle MFMA hides at most three other instructions:
   // everything an iteration needs (fragment read bases, request destinations and sources) is
   // therefore computed during the previous k-step in pieces of at most three instructions,
@@ -500,14 +559,14 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   unsigned oa = 0;                                             // A of tile t
   unsigned oa1 = 2 * S::kUnitBytes, ob1 = 3 * S::kUnitBytes;   // A, B of tile t+1
   unsigned rd_a1 = rdbase_a1, rd_b1 = rdbase_b1 + S::kUnitBytes;   // reads of (t, k-step 1)
-  unsigned req_a = lds_wave + 4 * S::kUnitBytes;                   // A of t+2
-  const char* src_a = k_src(a_tile, 2);
+  unsigned req_a = lds_wave + 2 * S::kAhead * S::kUnitBytes;       // A of t+kAhead
+  const char* src_a = k_src(a_tile, S::kAhead);
   unsigned rd_a0 = 0, rd_b0 = 0, req_b = 0;                        // set during k-step 0
   const char* src_b = b_tile;
   int kt = 0;
 #define TFK_PIN_S(x) asm volatile("" : "+s"(x))
 #define TFK_PIN_V(x) asm volatile("" : "+v"(x))
-  // pieces run in the gaps of slot kPrepSlot (and the one after it) of k-step 0 / k-step 1
+  // pieces run in the read-free gaps from slot kPrepSlot on of k-step 0 / k-step 1
   auto prep0 = [&](int step, int t) __attribute__((always_inline)) {
     __builtin_amdgcn_sched_barrier(0);
     switch (step) {
@@ -516,7 +575,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
       case 2: rd_a0 = rdbase_a0 + oa1; TFK_PIN_V(rd_a0); break;
       case 3: rd_b0 = rdbase_b0 + ob1; TFK_PIN_V(rd_b0); break;
       case 4: req_b = lds_wave + oa; TFK_PIN_S(req_b); break;
-      case 5: kt = t; TFK_PIN_S(kt); kt = min(kt + 2, last_tile); TFK_PIN_S(kt); break;
+      case 5: kt = t; TFK_PIN_S(kt); kt = min(kt + S::kAhead, last_tile); TFK_PIN_S(kt); break;
       case 6: src_b = b_tile + (size_t)(unsigned)(kt * (S::BK * 2)); TFK_PIN_S(src_b); break;
       default: break;
     }
@@ -527,21 +586,19 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     switch (step) {
       case 0: oa = oa1; TFK_PIN_S(oa); rd_a1 = rdbase_a1 + oa; TFK_PIN_V(rd_a1); break;
       case 1: rd_b1 = rdbase_b1 + ob1; TFK_PIN_V(rd_b1); break;
-      case 2: req_a = ring(oa + 4 * S::kUnitBytes); TFK_PIN_S(req_a); break;
+      case 2: req_a = ring(oa + 2 * S::kAhead * S::kUnitBytes); TFK_PIN_S(req_a); break;
       case 3: req_a += lds_wave; TFK_PIN_S(req_a); break;
-      case 4: kt = t; TFK_PIN_S(kt); kt = min(kt + 3, last_tile); TFK_PIN_S(kt); break;
+      case 4: kt = t; TFK_PIN_S(kt); kt = min(kt + S::kAhead + 1, last_tile); TFK_PIN_S(kt); break;
       case 5: src_a = a_tile + (size_t)(unsigned)(kt * (S::BK * 2)); TFK_PIN_S(src_a); break;
       default: break;
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  constexpr int kPrepSlot = 6;   // slots 6 and 7 carry no fragment reads
   // request n of a k-step goes at the head of slot n * kSlotsPerLoad; if n % 4 == 0 its M0 is
   // written in the last gap of the slot before (for slot 0: of the previous k-step's slot 7)
   auto m0_slot = [&](int i, int j, unsigned next_unit, unsigned this_unit) __attribute__((always_inline)) {
-    if (j != S::TN - 1) return;
+    if (j != S::TN - 1 || !S::m0_slot_after(i)) return;
     const int i_next = (i + 1) % S::TM;
-    if (i_next % kSlotsPerLoad != 0 || (i_next / kSlotsPerLoad) % 4 != 0) return;
     __builtin_amdgcn_sched_barrier(0);
     set_m0(i_next == 0 ? next_unit : this_unit, i_next / kSlotsPerLoad);
     __builtin_amdgcn_sched_barrier(0);
@@ -553,7 +610,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
       __builtin_amdgcn_sched_barrier(0);
       if (i % kSlotsPerLoad == 0) request(src_a, i / kSlotsPerLoad);
       slot_pinned(0, i, rd_a1, rd_b1, [&](int j) __attribute__((always_inline)) {
-        if (i >= kPrepSlot) prep0((i - kPrepSlot) * S::TN + j, t);
+        prep0(S::kPrep.piece[i * S::TN + j], t);
         m0_slot(i, j, req_b, req_a);
       });
     }
@@ -564,7 +621,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
       __builtin_amdgcn_sched_barrier(0);
       if (i % kSlotsPerLoad == 0) request(src_b, i / kSlotsPerLoad);
       slot_pinned(1, i, rd_a0, rd_b0, [&](int j) __attribute__((always_inline)) {
-        if (i >= kPrepSlot) prep1((i - kPrepSlot) * S::TN + j, t);
+        prep1(S::kPrep.piece[i * S::TN + j], t);
         m0_slot(i, j, req_a, req_b);
       });
     }
@@ -635,9 +692,12 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
 #define TFK_GEMM_R64_WAVES_N 2
 #endif
 
-template <typename OutT>
+
+using RingBig = Ring64Shape<256, TFK_GEMM_R64_WAVES_N, 2>;   // 5 units of 32 KiB
+using RingMid = Ring64Shape<128, 2, 4>;                      // 9 units of 16 KiB
+
+template <typename S, typename OutT>
 int launch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
-  using S = Ring64Shape<TFK_GEMM_R64_WAVES_N>;
   auto kern = gemm_ring64_kernel<S, OutT>;
   constexpr int lds = S::kUnits * S::kUnitBytes;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
@@ -770,10 +830,18 @@ int launch_guarded(const void* A, const void* B, void* C, int M, int N, int K, h
 
 template <typename OutT>
 int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
-#ifndef TFK_GEMM_NO_RING64
-  if (M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
-    return launch_ring64<OutT>(A, B, C, M, N, K, st);
-#endif
+  // 256 x 256 tiles do ~1.5x the work per cycle of 128 x 128 tiles (measured: 96 vs 146 us at
+  // 4096^3) but come in quarters as many: compare the rounds of tiles the 256 CUs need, a round
+  // of big tiles costing 4 units and a round of mid tiles 1.6.
+  if (M % 128 == 0 && N % 128 == 0 && K % 64 == 0) {
+    constexpr int64_t kCUs = 256;
+    const bool big_fits = M % 256 == 0 && N % 256 == 0;
+    const int64_t big_rounds = ((M / 256) * (N / 256) + kCUs - 1) / kCUs;
+    const int64_t mid_rounds = ((M / 128) * (N / 128) + kCUs - 1) / kCUs;
+    if (big_fits && 5 * big_rounds <= 2 * mid_rounds)
+      return launch_ring64<RingBig, OutT>(A, B, C, M, N, K, st);
+    return launch_ring64<RingMid, OutT>(A, B, C, M, N, K, st);
+  }
   if (M % 256 == 0 && N % 256 == 0 && K % ShapeBig::BK == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
     return launch_direct<ShapeBig, OutT>(A, B, C, M, N, K, st);
   if (M % 128 == 0 && N % 128 == 0 && K % 32 == 0)
