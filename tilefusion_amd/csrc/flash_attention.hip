@@ -169,35 +169,69 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   const int num_tiles = (n_end + kBN - 1) / kBN;
 
   // ---- global -> LDS plan: wavefront instruction i of a tile covers 1 KiB of it ------------
+  // Request r of a wavefront (r < kKPerWave: K tile, else V tile) is one instruction: scalar
+  // base (start of the tile in global memory) + a per-lane 32-bit offset computed once here.
+  // Only a tile that crosses the end of the keys takes the slow form with clamped addresses.
   const unsigned smem_base = lds_address(smem);
-  auto issue_tile_loads = [&](int tile) __attribute__((always_inline)) {
-    const int n0 = min(tile, num_tiles - 1) * kBN;  // clamped past the end (never read)
-    const unsigned sk = smem_base + (tile % kStages) * kStageBytes;
-    const unsigned sv = sk + kKBytes;
+  unsigned req_off[kLoadsPerTile];   // per-lane byte offset inside the tile (global side)
+  unsigned req_lds[kLoadsPerTile];   // wave-uniform byte offset inside the stage (LDS side)
 #pragma unroll
-    for (int t = 0; t < kKPerWave; ++t) {  // K tile: [kBN][D]
-      const int i = (wave + kWavesT * t) % kKInstr;
+  for (int t = 0; t < kKPerWave; ++t) {  // K tile: [kBN][D]
+    const int i = (wave + kWavesT * t) % kKInstr;
+    constexpr int kRowsPerInstr = 64 / kKChunks;
+    const int row = i * kRowsPerInstr + lane / kKChunks;
+    req_off[t] = (unsigned)(row * D + swz_k<kKChunks>(row, lane % kKChunks) * 8) * 2u;
+    req_lds[t] = i * 1024;
+  }
+#pragma unroll
+  for (int t = 0; t < kVPerWave; ++t) {
+    const int i = (wave + kWavesT * t) % kVInstr;
+    constexpr int kRowsPerInstr = 64 / kVChunks;
+    const int row = i * kRowsPerInstr + lane / kVChunks;
+    if constexpr (!kVT)  // V tile: [kBN][DV]
+      req_off[kKPerWave + t] = (unsigned)(row * DV + swz_v<kVChunks>(row, lane % kVChunks) * 8) * 2u;
+    else                 // V^T tile: [DV][kBN] out of a [DV][Lkv] matrix
+      req_off[kKPerWave + t] = ((unsigned)row * (unsigned)Lkv + swz_k<kVChunks>(row, lane % kVChunks) * 8) * 2u;
+    req_lds[kKPerWave + t] = kKBytes + i * 1024;
+  }
+  auto issue_request = [&](int tile, int r) __attribute__((always_inline)) {
+    const int n0 = min(tile, num_tiles - 1) * kBN;  // clamped past the end (never read)
+    const unsigned dst = smem_base + (tile % kStages) * kStageBytes + req_lds[r];
+    if (n0 + kBN <= Lkv) {
+      const char* base = r < kKPerWave ? reinterpret_cast<const char*>(K + (size_t)n0 * D)
+                         : kVT         ? reinterpret_cast<const char*>(V + n0)
+                                       : reinterpret_cast<const char*>(V + (size_t)n0 * DV);
+      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(req_off[r]), "s"(base), "s"(dst)
+                   : "memory");
+      return;
+    }
+    if (r < kKPerWave) {
+      const int i = (wave + kWavesT * r) % kKInstr;
       constexpr int kRowsPerInstr = 64 / kKChunks;
       const int row = i * kRowsPerInstr + lane / kKChunks;
       const int cc = swz_k<kKChunks>(row, lane % kKChunks);
       const int gr = min(n0 + row, Lkv - 1);
-      lds_dma_16B(K + (size_t)gr * D + cc * 8, sk + i * 1024);
-    }
-#pragma unroll
-    for (int t = 0; t < kVPerWave; ++t) {
-      const int i = (wave + kWavesT * t) % kVInstr;
+      lds_dma_16B(K + (size_t)gr * D + cc * 8, dst);
+    } else {
+      const int i = (wave + kWavesT * (r - kKPerWave)) % kVInstr;
       constexpr int kRowsPerInstr = 64 / kVChunks;
       const int row = i * kRowsPerInstr + lane / kVChunks;
-      if constexpr (!kVT) {  // V tile: [kBN][DV]
+      if constexpr (!kVT) {
         const int cc = swz_v<kVChunks>(row, lane % kVChunks);
         const int gr = min(n0 + row, Lkv - 1);
-        lds_dma_16B(V + (size_t)gr * DV + cc * 8, sv + i * 1024);
-      } else {  // V^T tile: [DV][kBN] out of a [DV][Lkv] matrix
+        lds_dma_16B(V + (size_t)gr * DV + cc * 8, dst);
+      } else {
         const int cc = swz_k<kVChunks>(row, lane % kVChunks);
         const int gc = min(n0 + cc * 8, Lkv - 8);
-        lds_dma_16B(V + (size_t)row * Lkv + gc, sv + i * 1024);
+        lds_dma_16B(V + (size_t)row * Lkv + gc, dst);
       }
     }
+  };
+  auto issue_tile_loads = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+    for (int r = 0; r < kLoadsPerTile; ++r) issue_request(tile, r);
   };
 
   // ---- LDS -> register plan -----------------------------------------------------------------
@@ -248,15 +282,22 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     l_run[qb] = 0.f;
   }
 
-  // Ring of kStages tiles.  Iteration `it` starts with the ring step: wait until tile it+1 has
-  // landed (only the loads of younger tiles stay in flight), meet the other wavefronts, then
-  // request tile it+kStages-1 into the stage of tile it-1, which nobody reads any more.  Tile
+  // Ring of kStages tiles.  Iteration `it` starts with the ring barrier: wait until tile it+1
+  // has landed (only the loads of younger tiles stay in flight) and meet the other wavefronts;
+  // after it the stage of tile it-1 is free and tile it+kStages-1 is requested into it.  Tile
   // it+1 is needed that early because the wavefronts of a workgroup run in two phases (below).
+  // The requests are NOT issued in one burst behind the barrier: eight wavefronts handing 32
+  // KiB of requests to the CU's one address unit at the same moment all stall in the issue
+  // queue with the matrix pipe idle (measured: ~500 of 4100 cycles per tile).  They ride along
+  // with the MFMAs of the next QK product instead, one request per reduction step.
 #pragma unroll
   for (int t = 0; t < kStages - 1; ++t) issue_tile_loads(t);
   barrier_keep_vmem<(kStages - 2) * kLoadsPerTile>();  // tile 0 has landed
-  auto ring_step = [&](int it) __attribute__((always_inline)) {
+  auto ring_barrier = [&]() __attribute__((always_inline)) {
     barrier_keep_vmem<(kStages - 3) * kLoadsPerTile>();
+  };
+  auto ring_step = [&](int it) __attribute__((always_inline)) {  // burst form, off the hot path
+    ring_barrier();
     issue_tile_loads(it + kStages - 1);
   };
   float4_t s[kKB][kQB];  // scores of the tile in flight (carried across iterations by late wavefronts)
@@ -293,7 +334,8 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   // ---- S^T = K Q'^T - m: s[kb][qb][r] = log2-scaled score of key 64*it + 16*kb + 4*lg + r
   //      against row lr of query block qb, minus that row's reference maximum.  Expects the
   //      fragments of step kk = 0 to be on their way into kf[0]. ---------------------------
-  auto qk_tile = [&](int it) __attribute__((always_inline)) {
+  //      req_tile >= 0: that tile's requests are issued between the reduction steps.
+  auto qk_tile = [&](int it, int req_tile) __attribute__((always_inline)) {
 #pragma unroll
     for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
@@ -301,6 +343,12 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
     for (int kk = 0; kk < kKK; ++kk) {
       if (kk + 1 < kKK) k_reads((kk + 1) & 1, it, kk + 1);
+      if (req_tile >= 0) {
+#pragma unroll
+        for (int r = 0; r < kLoadsPerTile; ++r)
+          if ((r * kKK) / kLoadsPerTile == kk) issue_request(req_tile, r);
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
@@ -426,30 +474,40 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   k_reads(0, 0, 0);
   if (!late) {
     for (; it < n_plain; ++it) {
-      ring_step(it);
-      qk_tile(it);
+      ring_barrier();
+      qk_tile(it, it + kStages - 1);
       softmax_tile(it, std::false_type{});
       pv_tile(it, it + 1);
     }
     for (; it < n_compute; ++it) {
-      ring_step(it);
-      qk_tile(it);
+      ring_barrier();
+      qk_tile(it, it + kStages - 1);
       softmax_tile(it, std::true_type{});
       pv_tile(it, it + 1);
     }
   } else {
-    qk_tile(0);
+    // The issue arbiter prefers the older wavefront: when this wavefront's QK product meets
+    // the first one's PV product on the MFMA pipe it would lose every slot, reach the barrier
+    // ~700 cycles after the first one (measured with s_memtime) and finish its product alone
+    // with the other wavefront idle.  Raised priority for that one product evens them out.
+    auto late_qk = [&](int it_) __attribute__((always_inline)) {
+      __builtin_amdgcn_s_setprio(2);
+      if (it_ + 1 < n_compute) qk_tile(it_ + 1, it_ + kStages - 1);
+      else issue_tile_loads(it_ + kStages - 1);
+      __builtin_amdgcn_s_setprio(0);
+    };
+    qk_tile(0, -1);
     for (; it < n_plain; ++it) {
-      ring_step(it);
+      ring_barrier();
       softmax_tile(it, std::false_type{});
       pv_tile(it, it + 1);
-      if (it + 1 < n_compute) qk_tile(it + 1);
+      late_qk(it);
     }
     for (; it < n_compute; ++it) {
-      ring_step(it);
+      ring_barrier();
       softmax_tile(it, std::true_type{});
       pv_tile(it, it + 1);
-      if (it + 1 < n_compute) qk_tile(it + 1);
+      late_qk(it);
     }
   }
   for (; it < num_tiles; ++it) ring_step(it);
