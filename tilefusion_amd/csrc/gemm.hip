@@ -688,13 +688,8 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   }
 }
 
-#ifndef TFK_GEMM_R64_WAVES_N
-#define TFK_GEMM_R64_WAVES_N 2
-#endif
-
-
-using RingBig = Ring64Shape<256, TFK_GEMM_R64_WAVES_N, 2>;   // 5 units of 32 KiB
-using RingMid = Ring64Shape<128, 2, 4>;                      // 9 units of 16 KiB
+using RingBig = Ring64Shape<256, 2, 2>;   // 5 units of 32 KiB
+using RingMid = Ring64Shape<128, 2, 4>;   // 9 units of 16 KiB
 
 template <typename S, typename OutT>
 int launch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
@@ -790,10 +785,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_guarded_kernel(
       }
 }
 
-#ifndef TFK_GEMM_BIG
-#define TFK_GEMM_BIG 256, 256, 32, 2, 2, 4
-#endif
-using ShapeBig = DirectShape<TFK_GEMM_BIG>;           // 4 x 32 KiB of LDS, 128x128 per wavefront
+using ShapeBig = DirectShape<256, 256, 32, 2, 2, 4>;         // 4 x 32 KiB of LDS, 128x128 per wavefront
 using ShapeMid = DirectShape<128, 128, 32, 2, 2, 4>;      // 4 x 16 KiB, 64x64 per wavefront
 using ShapeSmall = GemmShape<64, 64, 32, 2, 2, 1>;    // bounds-checked path
 
