@@ -169,8 +169,10 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
   for (int f = tid; f < kRowsPerBlock * kDChunks; f += kThreads) {
     const int row = f / kDChunks, c = f % kDChunks;
     if (m0 + row < M)
-      *reinterpret_cast<uint4_t*>(D + (size_t)(m0 + row) * P + p0 + c * 8) =
-          *reinterpret_cast<const uint4_t*>(sD + row * TP + c * 8);
+      // streaming store: D is written once and not read again here, and an ordinary store next to
+      // the operand reads costs this HBM-bound kernel 10% (6.40 -> 5.72 us at 16384 x 128^3)
+      __builtin_nontemporal_store(*reinterpret_cast<const uint4_t*>(sD + row * TP + c * 8),
+                                  reinterpret_cast<uint4_t*>(D + (size_t)(m0 + row) * P + p0 + c * 8));
   }
 }
 
@@ -301,8 +303,8 @@ __global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
   for (int f = tid; f < kRows * kDChunks; f += kWavesT * 64) {
     const int row = f / kDChunks, c = f % kDChunks;
     if (m0 + row < M)
-      *reinterpret_cast<uint4_t*>(D + (size_t)(m0 + row) * P + c * 8) =
-          *reinterpret_cast<const uint4_t*>(sD + row * P + c * 8);
+      __builtin_nontemporal_store(*reinterpret_cast<const uint4_t*>(sD + row * P + c * 8),
+                                  reinterpret_cast<uint4_t*>(D + (size_t)(m0 + row) * P + c * 8));
   }
 }
 
