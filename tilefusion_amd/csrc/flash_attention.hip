@@ -514,17 +514,46 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   wait_vmem_all();  // the clamped tail loads must not outlive the workgroup's LDS
 
   // ---- epilogue: O[m][16*db + 4*lg + r] = O^T / l ------------------------------------------
+  // A lane holds 4 consecutive head dims of row lr for every 16-wide block db.  Stored as they
+  // are, a store instruction writes 16 rows x 32 bytes with the four lanes of a row 16 lane
+  // ids apart, and the address unit only merges ADJACENT lanes: 64 accesses per instruction.
+  // The data is therefore re-dealt first, a pair of blocks (db, db+1) at a time: the 16-lane
+  // groups g and g^1 trade halves (v_permlane16_swap), after which groups 0/2 hold dims 0-7 /
+  // 8-15 of block db and groups 1/3 the same of block db+1, 16 bytes per lane; ds_bpermute then
+  // moves the 16 bytes of (row r, segment s) to lane 4*r + s, and four adjacent lanes store 64
+  // contiguous bytes of a row.
+  {
+    const int st_row = lane >> 2, st_seg = lane & 3;
+    // segment s of a row lives in group {0, 2, 1, 3}[s] after the swap
+    const int src_lane = st_row + 16 * (((st_seg & 1) << 1) | (st_seg >> 1));
 #pragma unroll
-  for (int qb = 0; qb < kQB; ++qb) {
-    const float inv = 1.f / quad_sum(l_run[qb]);
-    const int m_row = q_row0 + 16 * qb + lr;
-    if (m_row < Lq) {
+    for (int qb = 0; qb < kQB; ++qb) {
+      const float inv = 1.f / quad_sum(l_run[qb]);   // of this lane's own row lr
+      const int m_row = q_row0 + 16 * qb + st_row;   // the row this lane stores
+      half_t* o_lane = O + (size_t)m_row * DV + 8 * st_seg;
 #pragma unroll
-      for (int db = 0; db < kDB; ++db) {
-        half4_t out;
+      for (int db = 0; db < kDB; db += 2) {
+        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+        unsigned x[2], y[2];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) out[t] = (half_t)(o_acc[db][qb][t] * inv);
-        *reinterpret_cast<half4_t*>(O + (size_t)m_row * DV + db * 16 + 4 * lg) = out;
+        for (int d = 0; d < 2; ++d) {
+          const h2_t hx = {(half_t)(o_acc[db][qb][2 * d] * inv), (half_t)(o_acc[db][qb][2 * d + 1] * inv)};
+          const h2_t hy = {(half_t)(o_acc[db + 1][qb][2 * d] * inv), (half_t)(o_acc[db + 1][qb][2 * d + 1] * inv)};
+          x[d] = __builtin_bit_cast(unsigned, hx);
+          y[d] = __builtin_bit_cast(unsigned, hy);
+#if defined(__HIP_DEVICE_COMPILE__)
+          // x of the odd groups <-> y of the even groups
+          auto sw = __builtin_amdgcn_permlane16_swap(x[d], y[d], false, false);
+          x[d] = sw[0];
+          y[d] = sw[1];
+#endif
+        }
+        uint4_t v;
+        v[0] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)x[0]);
+        v[1] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)x[1]);
+        v[2] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)y[0]);
+        v[3] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)y[1]);
+        if (m_row < Lq) *reinterpret_cast<uint4_t*>(o_lane + 16 * db) = v;
       }
     }
   }
