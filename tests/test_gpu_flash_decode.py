@@ -21,7 +21,8 @@ def _slices(bh, lkv):
 
 
 @pytest.mark.parametrize("bh,lkv,splits", [(4, 1000, 3), (2, 777, 64), (3, 1, 1), (3, 5, 8), (8, 4096, 1),
-                                           (8, 4096, 64), (2, 32768, 64), (1, 20000, 7), (5, 128, 128)])
+                                           (8, 4096, 64), (2, 32768, 64), (1, 20000, 7), (5, 128, 128),
+                                           (2, 128, 1), (2, 256, 1), (2, 384, 1), (3, 129, 1), (3, 257, 2)])
 def test_shapes_and_ragged_splits(bh, lkv, splits):
     q, k, v = _slices(bh, lkv)
     o = c_decode(q.to(DEV), k.to(DEV), v.to(DEV), splits)
