@@ -194,8 +194,13 @@ int launch(const void* A, const void* B, const void* C, void* D, int batch, int 
 // n-tile; A fragments are loaded once.  A workgroup alone on a CU has to hide the L2 latency
 // with bytes in flight: two 64 KiB stages (one tile ahead) ran at a quarter of this speed.
 // ------------------------------------------------------------------------------------------
-template <int kWavesT>
-__global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
+// kSplit = 2: a second set of kWavesT wavefronts takes every other n-tile of the same rows (the
+// pair w, w + kWavesT shares a SIMD), and the two partial D tiles are added through LDS at the
+// end.  A wavefront's chain per tile - fragment reads, 16 MFMAs, fp16 conversion, 16 MFMAs that
+// depend on it - leaves the matrix pipe idle most of the time; a second, independent chain on
+// the same SIMD fills it.  Only the first set issues the tile requests.
+template <int kWavesT, int kSplit>
+__global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_kernel(
     const half_t* __restrict__ A, const half_t* __restrict__ B, const half_t* __restrict__ C,
     half_t* __restrict__ D, int M, int N) {
   constexpr int K = 128, P = 128, TN = 64, kStagesS = 4;
@@ -213,7 +218,9 @@ __global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   half_t* sD = reinterpret_cast<half_t*>(smem + kStagesS * kStageBytes);
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = wave_id % kWavesT;      // which 16 rows
+  const int half = wave_id / kWavesT;      // which n-tiles (t % kSplit == half)
   const int lr = lane & 15, lg = lane >> 4;
   const int m0 = blockIdx.x * kRows;
   const size_t batch = blockIdx.z;
@@ -240,6 +247,7 @@ __global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
   const unsigned voff_b0 = (lane / 16) * (K * 2) + (((lane % 16) ^ (lane / 16)) << 4);
   const unsigned voff_c0 = (lane / 8) * (unsigned)N * 2u + (((lane % 8) ^ (lane / 16)) << 4);
   auto request_tile = [&](int t) __attribute__((always_inline)) {
+    if (kSplit > 1 && half != 0) return;
     const unsigned stage = smem_base + (t % kStagesS) * kStageBytes;
     const int n0 = min(t, n_tiles - 1) * TN;
     const char* b_src = reinterpret_cast<const char*>(B) + (size_t)n0 * (K * 2);
@@ -284,6 +292,7 @@ __global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
     const char* sB = smem + (t % kStagesS) * kStageBytes;
     const char* sC = sB + kBBytes;
 
+    if (kSplit > 1 && t % kSplit != half) continue;
     float4_t acc1[TN / 16];
 #pragma unroll
     for (int nt = 0; nt < TN / 16; ++nt) acc1[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
@@ -291,16 +300,36 @@ __global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
     second_product<TN, P>(sC, acc1, acc2, lr, lg);
   }
   wait_vmem_all();  // the surplus requests must not outlive the workgroup's LDS
+  if constexpr (kSplit > 1) {
+    // add the second set's partial sums to the first set's (the ring is free by now)
+    __syncthreads();
+    constexpr int kPartElems = kWavesT * 8 * 64;   // float4 per wavefront set
+    static_assert((kSplit - 1) * kPartElems * 16 <= kStagesS * kStageBytes, "partial sums fit in the ring");
+    float4_t* part = reinterpret_cast<float4_t*>(smem) + (size_t)wave * 8 * 64 + lane;
+    if (half != 0) {
+#pragma unroll
+      for (int pt = 0; pt < 8; ++pt) part[(half - 1) * kPartElems + pt * 64] = acc2[pt];
+    }
+    __syncthreads();
+    if (half == 0) {
+#pragma unroll
+      for (int h = 1; h < kSplit; ++h)
+#pragma unroll
+        for (int pt = 0; pt < 8; ++pt) acc2[pt] += part[(h - 1) * kPartElems + pt * 64];
+    }
+  }
 
   // Epilogue: acc2[pt][r] = D[m0 + 16*wave + 4*lg + r][16*pt + lr], staged through LDS for
   // 16-byte stores along rows
+  if (half == 0) {
 #pragma unroll
-  for (int pt = 0; pt < 8; ++pt)
+    for (int pt = 0; pt < 8; ++pt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) sD[(wave * 16 + 4 * lg + r) * P + pt * 16 + lr] = (half_t)acc2[pt][r];
+      for (int r = 0; r < 4; ++r) sD[(wave * 16 + 4 * lg + r) * P + pt * 16 + lr] = (half_t)acc2[pt][r];
+  }
   __syncthreads();
   constexpr int kDChunks = P / 8;
-  for (int f = tid; f < kRows * kDChunks; f += kWavesT * 64) {
+  for (int f = tid; f < kRows * kDChunks; f += kWavesT * kSplit * 64) {
     const int row = f / kDChunks, c = f % kDChunks;
     if (m0 + row < M)
       __builtin_nontemporal_store(*reinterpret_cast<const uint4_t*>(sD + row * P + c * 8),
@@ -308,16 +337,16 @@ __global__ __launch_bounds__(kWavesT * 64) void fused_two_gemms_stream_kernel(
   }
 }
 
-template <int kWavesT>
+template <int kWavesT, int kSplit>
 int launch_stream(const void* A, const void* B, const void* C, void* D, int batch, int M, int N,
                   hipStream_t st) {
-  auto kern = fused_two_gemms_stream_kernel<kWavesT>;
+  auto kern = fused_two_gemms_stream_kernel<kWavesT, kSplit>;
   constexpr int lds = 4 * (64 * 128 * 2 + 128 * 64 * 2) + 16 * kWavesT * 128 * 2;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
   TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds));
   dim3 grid((M + 16 * kWavesT - 1) / (16 * kWavesT), 1, batch);
-  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * 64), lds, st, static_cast<const half_t*>(A),
+  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const half_t*>(A),
                      static_cast<const half_t*>(B), static_cast<const half_t*>(C),
                      static_cast<half_t*>(D), M, N);
   TFK_HIP_TRY(hipGetLastError());
@@ -363,7 +392,7 @@ extern "C" int tf_fused_two_gemms_f16(const void* A, const void* B, const void* 
   // long N: stream the B / C tiles through the LDS ring (8-15% faster than the plain kernel's
   // load - wait - multiply per n-tile; both are bound by the latencies of one wavefront per SIMD)
   if (K == 128 && P == 128 && N % 64 == 0 && N >= 256)
-    return launch_stream<4>(A, B, C, D, (int)batch, (int)M, (int)N, st);
+    return launch_stream<4, 2>(A, B, C, D, (int)batch, (int)M, (int)N, st);
   if (N % 128 == 0) return pick_tp<128>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
   return pick_tp<32>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
 }
