@@ -43,6 +43,23 @@ def test_shapes(m, n, k, p):
     assert N.rel_l2(d, ref) <= 1e-3 and N.max_abs(d, ref) <= 2e-2 * max(1.0, float(ref.abs().max()))
 
 
+# The streaming kernel (K = P = 128, N a multiple of 64 from 256 on): two wavefront sets take
+# alternate n-tiles and their partial sums are added at the end.  Tile counts that are even, odd
+# and not a multiple of the ring length; a ragged last row block; one row; a batch.  Operands are
+# small integers times a power of two, so both products, the fp16 rounding of the intermediate
+# and the final sums are exact and the comparison with the oracle is bit-exact.
+@pytest.mark.parametrize("batch,m,n", [(1, 64, 256), (1, 70, 320), (1, 1, 448), (1, 200, 1088), (3, 96, 384)])
+def test_streaming_kernel_exact(batch, m, n):
+    g = torch.Generator().manual_seed(17 * m + n + batch)
+    a = torch.randint(-2, 3, (batch, m, 128), generator=g).half()
+    b = (torch.randint(-2, 3, (batch, n, 128), generator=g) / 4).half()
+    c = (torch.randint(-2, 3, (batch, 128, n), generator=g) / 8).half()
+    d = c_fused(a.to(DEV), b.to(DEV), c.to(DEV)).cpu()
+    for i in range(batch):
+        ref = N.fused_two_gemms_ref_rounded(a[i], b[i], c[i])
+        assert torch.equal(d[i].float(), ref.half().float()), f"batch {i}"
+
+
 def test_batched():
     g = torch.Generator().manual_seed(4)
     a = (torch.randn(3, 192, 64, generator=g) / 8).half()
