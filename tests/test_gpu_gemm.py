@@ -95,7 +95,9 @@ def test_ring_kernel_exact(m, n, k, out_dtype):
 # 9 units, requests 4 tiles ahead): fewer k-tiles than the look-ahead, counts around the ring
 # length, one tile, non-square grids.
 @pytest.mark.parametrize("m,n,k", [(128, 128, 64), (128, 256, 128), (256, 128, 256), (384, 640, 320), (640, 384, 576),
-                                   (1024, 1024, 1216), (2048, 2048, 2048)])
+                                   (1024, 1024, 1216), (2048, 2048, 2048),
+                                   # more tiles than CUs: the 5-unit variant with two workgroups per CU
+                                   (2048, 2176, 64), (2176, 2048, 192), (2048, 2304, 448), (3072, 2560, 704)])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
 def test_ring_kernel_mid_tiles_exact(m, n, k, out_dtype):
     g = torch.Generator(device=DEV).manual_seed(m + 3 * n + 7 * k)
