@@ -83,6 +83,22 @@ TF_API int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void
                                int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
                                void* stream);
 
+/* tf_flash_decode_f16 without the workspace argument and without any allocation: the per-split
+ * partials live in a static device array inside the library (TF_FLASH_DECODE_STATIC_MAX_PARTIALS
+ * x (128 + 2) floats = 16.25 MiB, held by every GPU the library runs on until the process ends).
+ * No counterpart in the reference.  It is for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The device that
+ * owns `stream` must be current.  The first call on a device looks up the array's address there
+ * (hipGetSymbolAddress); no call allocates or frees.  batch_heads * num_splits above
+ * TF_FLASH_DECODE_STATIC_MAX_PARTIALS is rejected with TF_ERR_INVALID_ARG.  Same kernels and
+ * bit-identical results as tf_flash_decode_f16.  All calls on one GPU share the one array, so
+ * calls that overlap on a GPU (different streams, or threads) race: serialise them. */
+#define TF_FLASH_DECODE_STATIC_MAX_PARTIALS 32768 /* 512 (batch x head) slices x 64 splits */
+TF_API size_t tf_flash_decode_static_max_partials(void);
+TF_API int tf_flash_decode_static_f16(const void* Q, const void* K, const void* V, void* O,
+                                      int64_t batch_heads, int64_t Lkv, int64_t D, int num_splits,
+                                      double softmax_scale, void* stream);
+
 /* data[indices[i, 0..index_depth-1], ...] += updates[i, ...] for every index row i; duplicate
  * rows accumulate (atomic adds), rows that point outside `data` are skipped.  `data` has
  * `rank` dimensions data_dims (host array, row-major, contiguous); indices is a device

@@ -14,6 +14,8 @@
 //     stores (ordinary stores in the middle of the read stream cost 7% of its bandwidth);
 //   * combine kernel: grid batch_heads, 128 threads, merges the fp32 partials.
 // All offsets are 64-bit.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace tfk {
@@ -205,27 +207,29 @@ extern "C" size_t tf_flash_decode_workspace_bytes(int64_t batch_heads, int64_t D
   return (size_t)batch_heads * (size_t)num_splits * (size_t)(D + 2) * sizeof(float);
 }
 
-extern "C" int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void* O,
-                                   void* workspace, size_t workspace_bytes, int64_t batch_heads,
-                                   int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
-                                   void* stream) {
-  using namespace tfk;
-  TFK_REQUIRE(Q && K && V && O && workspace, TF_ERR_INVALID_ARG, "tf_flash_decode_f16: null pointer");
+namespace tfk {
+namespace {
+
+// Argument checks shared by both entry points.
+int check_decode_args(const char* who, const void* Q, const void* K, const void* V, const void* O,
+                      int64_t batch_heads, int64_t Lkv, int64_t D, int num_splits,
+                      double softmax_scale) {
+  TFK_REQUIRE(Q && K && V && O, TF_ERR_INVALID_ARG, "%s: null pointer", who);
   TFK_REQUIRE(batch_heads > 0 && Lkv > 0 && num_splits > 0, TF_ERR_INVALID_ARG,
-              "tf_flash_decode_f16: sizes must be positive");
+              "%s: sizes must be positive", who);
   TFK_REQUIRE(batch_heads < 65536 && num_splits <= 65536, TF_ERR_INVALID_ARG,
-              "tf_flash_decode_f16: batch_heads / num_splits too large");
-  TFK_REQUIRE(D == kD, TF_ERR_UNSUPPORTED, "tf_flash_decode_f16: head dim must be 128 (got %lld)",
-              (long long)D);
+              "%s: batch_heads / num_splits too large", who);
+  TFK_REQUIRE(D == kD, TF_ERR_UNSUPPORTED, "%s: head dim must be 128 (got %lld)", who, (long long)D);
   TFK_REQUIRE(softmax_scale == softmax_scale && softmax_scale - softmax_scale == 0.0,
-              TF_ERR_INVALID_ARG, "tf_flash_decode_f16: softmax_scale must be finite");
-  const size_t need = tf_flash_decode_workspace_bytes(batch_heads, D, num_splits);
-  TFK_REQUIRE(workspace_bytes >= need, TF_ERR_INVALID_ARG,
-              "tf_flash_decode_f16: workspace holds %zu bytes, %zu needed", workspace_bytes, need);
-  TFK_REQUIRE(((uintptr_t)workspace & 15) == 0, TF_ERR_INVALID_ARG,
-              "tf_flash_decode_f16: workspace must be 16-byte aligned");
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  float* o_part = static_cast<float*>(workspace);
+              TF_ERR_INVALID_ARG, "%s: softmax_scale must be finite", who);
+  return TF_OK;
+}
+
+// Split kernel + combine kernel on `st`; `partials` holds o_part then ml_part.
+int launch_decode(const void* Q, const void* K, const void* V, void* O, float* partials,
+                  int64_t batch_heads, int64_t Lkv, int num_splits, double softmax_scale,
+                  hipStream_t st) {
+  float* o_part = partials;
   float* ml_part = o_part + (size_t)batch_heads * num_splits * kD;
   const int64_t chunk = (Lkv + num_splits - 1) / num_splits;
   const float scale_log2 = (float)(softmax_scale * 1.4426950408889634);
@@ -238,4 +242,88 @@ extern "C" int tf_flash_decode_f16(const void* Q, const void* K, const void* V, 
                      o_part, ml_part, static_cast<half_t*>(O), num_splits);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
+}
+
+}  // namespace
+}  // namespace tfk
+
+extern "C" int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void* O,
+                                   void* workspace, size_t workspace_bytes, int64_t batch_heads,
+                                   int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
+                                   void* stream) {
+  using namespace tfk;
+  TFK_REQUIRE(workspace, TF_ERR_INVALID_ARG, "tf_flash_decode_f16: null pointer");
+  if (int rc = check_decode_args("tf_flash_decode_f16", Q, K, V, O, batch_heads, Lkv, D, num_splits,
+                                 softmax_scale))
+    return rc;
+  const size_t need = tf_flash_decode_workspace_bytes(batch_heads, D, num_splits);
+  TFK_REQUIRE(workspace_bytes >= need, TF_ERR_INVALID_ARG,
+              "tf_flash_decode_f16: workspace holds %zu bytes, %zu needed", workspace_bytes, need);
+  TFK_REQUIRE(((uintptr_t)workspace & 15) == 0, TF_ERR_INVALID_ARG,
+              "tf_flash_decode_f16: workspace must be 16-byte aligned");
+  return launch_decode(Q, K, V, O, static_cast<float*>(workspace), batch_heads, Lkv, num_splits,
+                       softmax_scale, static_cast<hipStream_t>(stream));
+}
+
+// ---- the same pair of kernels with the partials in a static device array -------------------
+//
+// For callers that cannot allocate device memory (code under HIP graph capture, tight serving
+// loops, harnesses that forbid hipMalloc): no workspace argument, nothing allocated.  Every GPU
+// the library runs on holds its own copy of `scratch` until the process ends.  The name
+// `scratch` is only a host-side handle of the symbol, not a device address: the address on each
+// device comes from hipGetSymbolAddress, once, with that device current, and only that pointer
+// is ever handed to a kernel.
+namespace tfk {
+namespace {
+
+constexpr size_t kScratchFloats = (size_t)TF_FLASH_DECODE_STATIC_MAX_PARTIALS * (kD + 2);
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int scratch_on_current_device(float** out) {
+  int dev = -1;
+  TFK_HIP_TRY(hipGetDevice(&dev));
+  TFK_REQUIRE(dev >= 0 && dev < kMaxDevices, TF_ERR_UNSUPPORTED,
+              "tf_flash_decode_static_f16: device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    TFK_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    TFK_REQUIRE(p != nullptr, TF_ERR_HIP, "tf_flash_decode_static_f16: null symbol address");
+    g_scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return TF_OK;
+}
+
+}  // namespace
+}  // namespace tfk
+
+extern "C" size_t tf_flash_decode_static_max_partials(void) {
+  return (size_t)TF_FLASH_DECODE_STATIC_MAX_PARTIALS;
+}
+
+extern "C" int tf_flash_decode_static_f16(const void* Q, const void* K, const void* V, void* O,
+                                          int64_t batch_heads, int64_t Lkv, int64_t D,
+                                          int num_splits, double softmax_scale, void* stream) {
+  using namespace tfk;
+  if (int rc = check_decode_args("tf_flash_decode_static_f16", Q, K, V, O, batch_heads, Lkv, D,
+                                 num_splits, softmax_scale))
+    return rc;
+  TFK_REQUIRE((uint64_t)batch_heads * (uint64_t)num_splits <= TF_FLASH_DECODE_STATIC_MAX_PARTIALS,
+              TF_ERR_INVALID_ARG,
+              "tf_flash_decode_static_f16: batch_heads * num_splits = %llu exceeds the static "
+              "scratch array (%llu partials); use tf_flash_decode_f16 with a workspace",
+              (unsigned long long)((uint64_t)batch_heads * (uint64_t)num_splits),
+              (unsigned long long)TF_FLASH_DECODE_STATIC_MAX_PARTIALS);
+  float* partials = nullptr;
+  if (int rc = scratch_on_current_device(&partials)) return rc;
+  // Nothing has to start at zero: the split kernel writes every (slice, split) partial the
+  // combine kernel reads, so whatever an earlier call left in the array is never read.
+  return launch_decode(Q, K, V, O, partials, batch_heads, Lkv, num_splits, softmax_scale,
+                       static_cast<hipStream_t>(stream));
 }
