@@ -217,7 +217,7 @@ class Attention:
                 oracle.attention_ref(q[b, h], k[b, h], v[b, h], causal=self.causal)
         t = _cpu_time(run, reps=2)
         return {"value": self.flops * n / 64 / t / 1e12, "unit": "TFLOP/s",
-                "sample": "%d of 64 (batch, head) slices, fp32 softmax(QK^T)V per slice, best of 2" % n}
+                "sample": "extrapolated from %d of 64 (batch, head) slices (rate = sampled flops / sampled time), fp32 softmax(QK^T)V per slice, best of 2" % n}
 
 
 class Decode:
@@ -268,7 +268,7 @@ class Decode:
                 oracle.flash_decode_ref(q, k, v)
         t = _cpu_time(run)
         return {"value": self.bytes * len(host) / self.BH / t / 1e9, "unit": "GB/s",
-                "sample": "%d of 512 (batch, head) slices, fp32 softmax(qK^T)V per slice, best of 3" % len(host)}
+                "sample": "extrapolated from %d of 512 (batch, head) slices (rate = sampled bytes / sampled time), fp32 softmax(qK^T)V per slice, best of 3" % len(host)}
 
     config = {"workload": "flash-decoding fp16 B=16 H=32 q_len=1 KV=32768 D=128, 64 splits + LSE combine (2 kernels per step)",
               "inputs": "N(0,1) drawn on the device, seed 1005; 8 GiB of K,V (exceeds the last-level cache)"}

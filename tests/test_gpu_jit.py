@@ -11,6 +11,23 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+@pytest.fixture(autouse=True, scope="module")
+def fresh_disk_cache(tmp_path_factory):
+    """Compile into an empty directory so that no code object left by an earlier build of the
+    library can be picked up."""
+    import os
+    from tilefusion_amd.jit import JitCompiler
+    old = os.environ.get("TILEFUSION_CACHE_DIR")
+    os.environ["TILEFUSION_CACHE_DIR"] = str(tmp_path_factory.mktemp("jit_cache"))
+    JitCompiler.clear_cache()
+    yield
+    JitCompiler.clear_cache()
+    if old is None:
+        os.environ.pop("TILEFUSION_CACHE_DIR", None)
+    else:
+        os.environ["TILEFUSION_CACHE_DIR"] = old
+
+
 def test_jit_vector_add():
     from tilefusion_amd.jit import JitCompiler
     from tests.test_jit_cpu import ADD_SRC

@@ -65,3 +65,52 @@ def test_wrappers_validate_before_compiling(cache_dir):
     with pytest.raises(ValueError, match="must be a cuda tensor"):
         jit.fused_two_gemms_jit(t, t, t, t)
     assert not glob.glob(os.path.join(str(cache_dir), "*"))
+
+
+def test_cache_key_covers_the_contents_of_included_headers(cache_dir, tmp_path_factory):
+    # Same source, same include path, edited header: a second code object, not a stale hit.
+    from tilefusion_amd.jit import JitCompiler
+    inc = tmp_path_factory.mktemp("inc")
+    src = '#include "k.hpp"\nextern "C" __global__ void scale_kernel(float* x) { x[threadIdx.x] *= kFactor; }'
+
+    def compile_with(factor):
+        (inc / "k.hpp").write_text(f"constexpr float kFactor = {factor}f;\n")
+        try:
+            JitCompiler.get_or_compile_kernel("scale_kernel", src, [str(inc)])
+        except RuntimeError as e:
+            assert not torch.cuda.is_available() and "hipModuleLoadData" in str(e)
+
+    compile_with(2.0)
+    assert len(glob.glob(os.path.join(str(cache_dir), "*.hsaco"))) == 1
+    # the digest of a directory is taken once per process; a new process sees the edit, which
+    # is what a library update between runs looks like.  Emulate it with a second directory
+    # of the same contents but the edited header.
+    inc2 = tmp_path_factory.mktemp("inc2")
+    (inc2 / "k.hpp").write_text("constexpr float kFactor = 3.0f;\n")
+    try:
+        JitCompiler.get_or_compile_kernel("scale_kernel", src, [str(inc2)])
+    except RuntimeError as e:
+        assert not torch.cuda.is_available() and "hipModuleLoadData" in str(e)
+    assert len(glob.glob(os.path.join(str(cache_dir), "*.hsaco"))) == 2
+
+
+def test_kernel_handles_die_with_clear_cache():
+    from tilefusion_amd.jit import JitCompiler, Kernel
+    k = Kernel(0, "stale")
+    JitCompiler.clear_cache()
+    with pytest.raises(RuntimeError, match="unloaded by JitCompiler.clear_cache"):
+        k.launch((1,), (64,), ())
+
+
+def test_attention_kernel_name_is_stable_across_processes():
+    # the name is part of the source and therefore of the disk-cache key: it must not depend
+    # on Python's per-process string hashing
+    import struct
+    import subprocess
+    import sys
+    code = "import struct; print(struct.pack('<d', 0.08838834764831845).hex())"
+    outs = {subprocess.check_output([sys.executable, "-c", code], env={**os.environ, "PYTHONHASHSEED": str(s)}) for s in (1, 2)}
+    assert len(outs) == 1
+    import inspect
+    from tilefusion_amd import jit
+    assert "hash(" not in inspect.getsource(jit.flash_attention_jit)

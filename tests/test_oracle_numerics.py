@@ -63,6 +63,16 @@ def test_fused_ref_hand_case_and_rounding_bound():
     assert N.rel_l2(dr, d) < 5e-4  # the fp16 intermediate costs < half the tolerance
 
 
+def test_fused_ref_rounded_rounds_the_intermediate_to_fp16():
+    # A@B = [2049, 4099]: 2049 is a tie between the fp16 neighbours 2048 and 2050 (-> even, 2048),
+    # 4099 lies between 4096 and 4100 (-> 4100).  Without the rounding D would be 2049 / 4099.
+    a = torch.tensor([[2048., 1.], [4096., 3.]]).half()
+    b = torch.tensor([[1., 1.]]).half()                 # N = 1, K = 2
+    c = torch.tensor([[1.], [0.5]]).half()              # P = 2, N = 1
+    assert N.fused_two_gemms_ref(a, b, c).tolist() == [[2049., 1024.5], [4099., 2049.5]]
+    assert N.fused_two_gemms_ref_rounded(a, b, c).tolist() == [[2048., 1024.], [4100., 2050.]]
+
+
 def test_attention_ref_invariants():
     g = torch.Generator().manual_seed(7)
     q = torch.randn(3, 16, 8, generator=g).half()

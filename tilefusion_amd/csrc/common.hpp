@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -92,6 +93,22 @@ int hip_fail(hipError_t e, const char* what);
   do {                                                      \
     hipError_t e__ = (expr);                                \
     if (e__ != hipSuccess) return ::tfk::hip_fail(e__, #expr); \
+  } while (0)
+
+// Opts `kern` in to `lds` bytes of dynamic LDS.  The attribute is per device and sticky, so the
+// runtime call is made once per kernel and device (a bit per device ordinal in a static of the
+// calling template instantiation, i.e. of the kernel), not on every launch.
+#define TFK_LDS_OPT_IN(kern, lds)                                                              \
+  do {                                                                                         \
+    static std::atomic<unsigned long long> done__{0};                                          \
+    int dev__ = 0;                                                                             \
+    TFK_HIP_TRY(hipGetDevice(&dev__));                                                         \
+    const unsigned long long bit__ = (dev__ >= 0 && dev__ < 64) ? (1ull << dev__) : 0ull;      \
+    if (!(done__.load(std::memory_order_acquire) & bit__) || bit__ == 0) {                     \
+      TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                     \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (lds)));     \
+      done__.fetch_or(bit__, std::memory_order_release);                                       \
+    }                                                                                          \
   } while (0)
 
 #define TFK_REQUIRE(cond, code, ...)  \

@@ -568,8 +568,7 @@ int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, in
   auto kern = flash_attention_fwd_kernel<D, DV, kVT, kCausal, kWavesT, kQB>;
   constexpr int lds = kStages * (kBN * D * 2 + kBN * DV * 2);
   static_assert(lds <= kMaxLdsBytes, "tiles do not fit in LDS");
-  TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  TFK_LDS_OPT_IN(kern, lds);
   constexpr int bm = kWavesT * 16 * kQB;
   const int q_tiles = (Lq + bm - 1) / bm;
   // causal with an even tile count: one workgroup per PAIR of query tiles (see the kernel)
@@ -586,10 +585,7 @@ int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, in
 template <int D, int DV, bool kVT, bool kCausal>
 int launch(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
            float scale_log2, hipStream_t st) {
-#ifndef TFK_FA_BIG
-#define TFK_FA_BIG 8, 2
-#endif
-  if (Lq > 128) return launch_w<D, DV, kVT, kCausal, TFK_FA_BIG>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+  if (Lq > 128) return launch_w<D, DV, kVT, kCausal, 8, 2>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
   return launch_w<D, DV, kVT, kCausal, 4, 2>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
 }
 

@@ -343,8 +343,7 @@ int launch_stream(const void* A, const void* B, const void* C, void* D, int batc
   auto kern = fused_two_gemms_stream_kernel<kWavesT, kSplit>;
   constexpr int lds = 4 * (64 * 128 * 2 + 128 * 64 * 2) + 16 * kWavesT * 128 * 2;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
-  TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+  TFK_LDS_OPT_IN(kern, lds);
   dim3 grid((M + 16 * kWavesT - 1) / (16 * kWavesT), 1, batch);
   hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const half_t*>(A),
                      static_cast<const half_t*>(B), static_cast<const half_t*>(C),

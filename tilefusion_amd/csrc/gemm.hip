@@ -697,14 +697,7 @@ int launch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hi
   auto kern = gemm_ring64_kernel<S, OutT>;
   constexpr int lds = S::kUnits * S::kUnitBytes;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
-  static thread_local int configured_dev = -1;
-  int dev = 0;
-  TFK_HIP_TRY(hipGetDevice(&dev));
-  if (configured_dev != dev) {
-    TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    configured_dev = dev;
-  }
+  TFK_LDS_OPT_IN(kern, lds);
   const int tiles_m = M / S::BM, tiles_n = N / S::BN;
   hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(S::kThreads), lds, st,
                      static_cast<const half_t*>(A), static_cast<const half_t*>(B),
@@ -795,14 +788,7 @@ int launch_direct(const void* A, const void* B, void* C, int M, int N, int K, hi
   auto kern = gemm_direct_lds_kernel<S, OutT>;
   constexpr int lds = S::kStages * S::kStageBytes;
   static_assert(lds <= kMaxLdsBytes, "tile does not fit in LDS");
-  static thread_local int configured_dev = -1;
-  int dev = 0;
-  TFK_HIP_TRY(hipGetDevice(&dev));
-  if (configured_dev != dev) {
-    TFK_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    configured_dev = dev;
-  }
+  TFK_LDS_OPT_IN(kern, lds);
   const int tiles_m = M / S::BM, tiles_n = N / S::BN;
   hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(S::kThreads), lds, st,
                      static_cast<const half_t*>(A), static_cast<const half_t*>(B),

@@ -1,12 +1,15 @@
 // Run-time compiler: implementation of tilefusion::jit::JitCompiler and its C ABI.
 // Counterpart of src/jit/compiler.cc:123-278 (popen(nvcc -ptx) -> cuModuleLoadData); here
 // popen(hipcc --genco) -> hipModuleLoadData, with a content-addressed disk cache.
+#include <dirent.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
 #include <cstdio>
 #include <cstdlib>
+#include <algorithm>
 #include <fstream>
+#include <map>
 #include <sstream>
 
 #include "common.hpp"
@@ -26,6 +29,42 @@ std::string hash_hex(const std::string& s) {
   char buf[17];
   snprintf(buf, sizeof(buf), "%016llx", h);
   return buf;
+}
+
+// Digest of every regular file below `dir` (relative name + contents, names sorted): a header
+// edited after a code object was cached must change the cache key.  Bounded in depth and file
+// count so that a stray include path (say "/") cannot stall a compile.
+void collect_files(const std::string& dir, const std::string& rel, int depth, std::vector<std::string>& out) {
+  if (depth > 6 || out.size() > 4096) return;
+  DIR* d = opendir((dir + "/" + rel).c_str());
+  if (!d) return;
+  std::vector<std::string> names;
+  while (dirent* e = readdir(d)) {
+    const std::string n = e->d_name;
+    if (n != "." && n != "..") names.push_back(n);
+  }
+  closedir(d);
+  std::sort(names.begin(), names.end());
+  for (const auto& n : names) {
+    const std::string r = rel.empty() ? n : rel + "/" + n;
+    struct stat st;
+    if (stat((dir + "/" + r).c_str(), &st) != 0) continue;
+    if (S_ISDIR(st.st_mode)) collect_files(dir, r, depth + 1, out);
+    else if (S_ISREG(st.st_mode) && out.size() <= 4096) out.push_back(r);
+  }
+}
+
+std::string directory_digest(const std::string& dir) {
+  std::vector<std::string> files;
+  collect_files(dir, "", 0, files);
+  std::string material;
+  for (const auto& r : files) {
+    std::ifstream f(dir + "/" + r, std::ios::binary);
+    std::stringstream ss;
+    ss << f.rdbuf();
+    material += r + "\n" + hash_hex(ss.str()) + "\n";
+  }
+  return hash_hex(material);
 }
 
 bool file_exists(const std::string& p) {
@@ -56,6 +95,27 @@ std::string hipcc_path() {
   return "/opt/rocm/bin/hipcc";
 }
 
+// What identifies the toolchain and this library in a cache key: the compiler's path, size and
+// modification time (a ROCm update replaces the file) and the library version.
+std::string toolchain_digest() {
+  const std::string cc = hipcc_path();
+  struct stat st;
+  std::ostringstream m;
+  m << cc << '\n' << tf_version() << '\n';
+  char resolved[4096];
+  const char* real = realpath(cc.c_str(), resolved);
+  if (real && stat(real, &st) == 0) m << real << '\n' << (long long)st.st_size << '\n' << (long long)st.st_mtime;
+  return hash_hex(m.str());
+}
+
+// A private directory: created with mode 0700, owned by this user, not writable by anyone else.
+bool private_dir_ok(const std::string& dir) {
+  if (mkdir(dir.c_str(), 0700) != 0 && errno != EEXIST) return false;
+  struct stat st;
+  if (lstat(dir.c_str(), &st) != 0 || !S_ISDIR(st.st_mode)) return false;
+  return st.st_uid == geteuid() && (st.st_mode & (S_IWGRP | S_IWOTH)) == 0;
+}
+
 }  // namespace
 
 JitCompiler& JitCompiler::instance() {
@@ -69,7 +129,17 @@ std::string JitCompiler::cache_dir() {
     const std::string dir = std::string(home) + "/.cache/tilefusion_mi355x";
     if (make_dirs(dir) && access(dir.c_str(), W_OK) == 0) return dir;
   }
-  return "/tmp/tilefusion_mi355x";
+  // No usable home directory: a per-user directory under /tmp, accepted only if it is ours and
+  // nobody else can write into it (a code object found there is loaded and run); failing
+  // that, a fresh directory that lives as long as the process and is never re-used.
+  const std::string shared = "/tmp/tilefusion_mi355x-" + std::to_string((long)geteuid());
+  if (private_dir_ok(shared)) return shared;
+  static const std::string fresh = [] {
+    char tmpl[] = "/tmp/tilefusion_mi355x-XXXXXX";
+    const char* d = mkdtemp(tmpl);
+    return std::string(d ? d : "");
+  }();
+  return fresh;
 }
 
 std::string JitCompiler::last_log() {
@@ -81,7 +151,7 @@ std::string JitCompiler::compile_to_code_object(const std::string& key, const st
                                                 const std::vector<std::string>& include_paths,
                                                 const std::vector<std::string>& compile_args) {
   const std::string dir = cache_dir();
-  if (!make_dirs(dir)) {
+  if (dir.empty() || !make_dirs(dir)) {
     last_log_ = "cannot create cache directory " + dir;
     return "";
   }
@@ -164,12 +234,21 @@ hipFunction_t JitCompiler::compile_kernel(const std::string& kernel_name, const 
   includes.insert(includes.end(), include_paths.begin(), include_paths.end());
   std::vector<std::string> args = get_default_compile_args();
   args.insert(args.end(), compile_args.begin(), compile_args.end());
-  std::string material = hip_source;
-  for (const auto& p : includes) material += "\n-I" + p;
+  std::lock_guard<std::mutex> lock(mutex_);
+  // The key covers everything the code object depends on: the source, the arguments, the
+  // CONTENTS of the include directories (digested once per process and directory) and the
+  // compiler and library versions.
+  static const std::string toolchain = toolchain_digest();
+  static std::map<std::string, std::string> dir_digests;
+  std::string material = hip_source + "\n" + toolchain;
+  for (const auto& p : includes) {
+    auto it = dir_digests.find(p);
+    if (it == dir_digests.end()) it = dir_digests.emplace(p, directory_digest(p)).first;
+    material += "\n-I" + p + "=" + it->second;
+  }
   for (const auto& a : args) material += "\n" + a;
   const std::string key = hash_hex(material);
 
-  std::lock_guard<std::mutex> lock(mutex_);
   const std::string cache_key = key + ":" + kernel_name;
   auto it = kernel_cache_.find(cache_key);
   if (it != kernel_cache_.end()) return it->second;

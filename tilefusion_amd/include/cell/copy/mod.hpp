@@ -1,3 +1,7 @@
+// Umbrella header of the copy primitives.
+// The list of headers and their names follow microsoft/TileFusion (MIT License,
+// Copyright (c) Microsoft Corporation), include/cell/copy/mod.hpp:6-14;
+// everything they include is written for gfx950.
 #pragma once
 
 #include "cell/copy/constants.hpp"

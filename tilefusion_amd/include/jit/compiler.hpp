@@ -4,8 +4,9 @@
 // Same contract as the reference: source text + kernel name (an `extern "C" __global__`
 // symbol) -> a launchable function handle, cached per process under a mutex.  What differs:
 //   * the compiler is `hipcc --genco` (a gfx950 code object), loaded with hipModuleLoadData;
-//   * the code object is also cached on disk, keyed by a hash of (source, include paths,
-//     arguments): the reference writes randomly named files it never re-uses;
+//   * the code object is also cached on disk, keyed by a hash of the source, the arguments,
+//     the contents of the include directories and the compiler / library versions: the
+//     reference writes randomly named files it never re-uses;
 //   * failure returns nullptr and keeps the compiler's output in last_log() instead of
 //     only logging it.
 #pragma once
@@ -40,7 +41,8 @@ class JitCompiler {
   std::string last_log();
 
   // Directory of the on-disk cache ($TILEFUSION_CACHE_DIR, else ~/.cache/tilefusion_mi355x,
-  // else /tmp/tilefusion_mi355x).
+  // else /tmp/tilefusion_mi355x-<uid> if that is a private directory of this user, else a
+  // fresh temporary directory of this process).
   static std::string cache_dir();
 
  private:

@@ -1,4 +1,7 @@
-// Umbrella header of the tile types (counterpart of include/types/mod.hpp:6-16).
+// Umbrella header of the tile types.
+// The list of headers and their names follow microsoft/TileFusion (MIT License,
+// Copyright (c) Microsoft Corporation), include/types/mod.hpp:6-16;
+// everything they include is written for gfx950.
 #pragma once
 
 #include "types/base.hpp"

@@ -13,6 +13,7 @@ tiling that was asked for.
 import ctypes
 import math
 import os
+import struct
 from typing import Sequence
 
 import torch
@@ -35,9 +36,12 @@ class Kernel:
 
     def __init__(self, handle: int, name: str):
         self._handle, self.name = handle, name
+        self._generation = JitCompiler._generation
 
     def launch(self, grid: Sequence[int], block: Sequence[int], args: Sequence, shared_mem: int = 0,
                stream=None) -> None:
+        if self._generation != JitCompiler._generation:
+            raise RuntimeError(f"kernel {self.name} was unloaded by JitCompiler.clear_cache(); compile it again")
         lib = _capi.load()
         boxed = []
         for a in args:
@@ -60,6 +64,10 @@ class Kernel:
 class JitCompiler:
     """Mirror of tilefusion::jit::JitCompiler (a process-wide singleton in the library)."""
 
+    # clear_cache() unloads the modules, which kills every function handle handed out so far:
+    # Kernel objects remember the generation they were made in and refuse to launch afterwards.
+    _generation = 0
+
     @staticmethod
     def get_or_compile_kernel(kernel_name: str, source: str, include_paths: Sequence[str] = (),
                               compile_args: Sequence[str] = ()) -> Kernel:
@@ -79,6 +87,7 @@ class JitCompiler:
 
     @staticmethod
     def clear_cache() -> None:
+        JitCompiler._generation += 1
         _capi.load().tf_jit_clear_cache()
 
     @staticmethod
@@ -160,7 +169,7 @@ def flash_attention_jit(q, k, v_t, o, tile_length_q=64, tile_length_kv=64, tile_
         raise ValueError("tile sizes must divide the problem")
     scale = 1.0 / math.sqrt(d) if softmax_scale is None else float(softmax_scale)
     wr, wc = warp_layout
-    tag = f"{lq}_{lkv}_{d}_{dv}_{tile_length_q}_{tile_length_kv}_{tk_}_{tp_}_{int(causal)}_{wr}_{abs(hash(repr(scale))) % 10**8}"
+    tag = f"{lq}_{lkv}_{d}_{dv}_{tile_length_q}_{tile_length_kv}_{tk_}_{tp_}_{int(causal)}_{wr}_{struct.pack('<d', float(scale)).hex()}"
     name = f"flash_attention_kernel_{tag}"
     src = _PRELUDE + f"""
 using Config = FlashAttentionTraits<__half, float, __half, TileShape<{lq}, {lkv}, {d}, {dv}>,
