@@ -282,7 +282,7 @@ TT_API int tt_atom_gemm(int variant, const void* a, const void* b, void* c) {
 
 // ---- 4. ke_gemm composed from the primitives (test_gemm.cu:172-215,316-375) ------------------
 template <typename Traits, typename AccType>
-__global__ void k_ke_gemm(const __half* a, const __half* b, AccType* c) {
+__global__ __launch_bounds__(Traits::kThreads) void k_ke_gemm(const __half* a, const __half* b, AccType* c) {
   kernels::ke_gemm<__half, AccType, Traits>(a, b, c);
 }
 template <typename WarpLayout, typename AccType, int M, int N, int K, int TM, int TN, int TK, int RK, int Stages, int Bytes>
@@ -373,7 +373,7 @@ TT_API int tt_softmax_pieces(int variant, const void* in, void* row_max, void* r
 // ---- 6. fused back-to-back GEMM composed from the primitives (tests/python/test_fused_two_gemms.py:
 //         M, N, K, P = 256, 128, 64, 64 with 64-wide tiles) ------------------------------------------
 template <typename Traits>
-__global__ void k_ke_fused(const __half* a, const __half* b, const __half* c, __half* d) {
+__global__ __launch_bounds__(Traits::kThreads) void k_ke_fused(const __half* a, const __half* b, const __half* c, __half* d) {
   kernels::ke_fused_two_gemms<__half, float, Traits>(a, b, c, d);
 }
 template <typename WarpLayout, int B, int M, int N, int K, int P, int TM, int TN, int TK, int TP>
@@ -404,7 +404,7 @@ TT_API void tt_ke_fused_shape(int variant, int* batch, int* m, int* n, int* k, i
 // ---- 7. flash attention composed from the primitives (tests/python/test_flash_attn.py:
 //         (64,128,128,128) plain and (128,128,128,128) causal, tiles (64,128,128,128), 4 wavefronts) ---
 template <typename Traits>
-__global__ void k_ke_flash(const __half* q, const __half* k, const __half* v, __half* o) {
+__global__ __launch_bounds__(Traits::kThreads) void k_ke_flash(const __half* q, const __half* k, const __half* v, __half* o) {
   kernels::ke_flash_attention<__half, float, __half, Traits>(q, k, v, o);
 }
 template <typename WarpLayout, int B, int M, int N, int K, int P, int TM, int TN, int TK, int TP, bool kCausal>
@@ -436,4 +436,337 @@ TT_API int tt_ke_flash(int variant, const void* q, const void* k, const void* v,
 TT_API void tt_ke_flash_shape(int variant, int* batch, int* m, int* n, int* k, int* p, int* causal) {
   const int* t = kFlashShapes[variant];
   *batch = t[0]; *m = t[1]; *n = t[2]; *k = t[3]; *p = t[4]; *causal = t[5];
+}
+
+// ---- 8. the pipelined GEMMs: Pipeline global -> LDS with asynchronous copies (level 1) plus a
+//         register-level Pipeline (level 2); tests/python/test_gemm.py:75-135 cases and more ----
+template <typename Traits, typename AccType, int kLevel>
+__global__ __launch_bounds__(Traits::kThreads) void k_ke_gemm_pipe(const __half* a, const __half* b, AccType* c) {
+  if constexpr (kLevel == 1) kernels::ke_gemm_level1_pipeline<__half, AccType, Traits>(a, b, c);
+  else kernels::ke_gemm_level2_pipeline<__half, AccType, Traits>(a, b, c);
+}
+template <typename WarpLayout, typename AccType, int kLevel, int M, int N, int K, int TM, int TN, int TK, int RK,
+          int Stages, int Bytes>
+static int run_ke_gemm_pipe(const void* a, const void* b, void* c) {
+  using Traits = kernels::KeGemmTraits<__half, AccType, WarpLayout, M, N, K, TM, TN, TK, RK, Stages, Bytes>;
+  auto kern = k_ke_gemm_pipe<Traits, AccType, kLevel>;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          Traits::kPipelineSharedBytes) != hipSuccess)
+    return -2;
+  hipLaunchKernelGGL(kern, dim3(M / TM, N / TN), dim3(Traits::kThreads), Traits::kPipelineSharedBytes, 0,
+                     static_cast<const __half*>(a), static_cast<const __half*>(b), static_cast<AccType*>(c));
+  return launch_status();
+}
+static const int kPipeShapes[9][4] = {{128, 128, 128, 0}, {256, 256, 256, 0}, {256, 256, 256, 0}, {512, 512, 512, 0},
+                                      {256, 256, 512, 0}, {128, 128, 256, 0}, {256, 256, 512, 1}, {128, 128, 384, 0},
+                                      {512, 256, 1024, 0}};
+TT_API int tt_ke_gemm_pipe(int variant, const void* a, const void* b, void* c) {
+  switch (variant) {
+    // the reference's own cases 1-4 (64 x 64 x 64 tiles; level 1 with 2 slots, level 2 with 3)
+    case 0: return run_ke_gemm_pipe<tl::RowMajor<2, 2>, float, 1, 128, 128, 128, 64, 64, 64, 32, 2, 64>(a, b, c);
+    case 1: return run_ke_gemm_pipe<tl::RowMajor<2, 2>, float, 1, 256, 256, 256, 64, 64, 64, 32, 2, 64>(a, b, c);
+    case 2: return run_ke_gemm_pipe<tl::RowMajor<2, 2>, float, 2, 256, 256, 256, 64, 64, 64, 32, 3, 64>(a, b, c);
+    case 3: return run_ke_gemm_pipe<tl::RowMajor<2, 2>, float, 2, 512, 512, 512, 64, 64, 64, 32, 3, 64>(a, b, c);
+    // level 1 with three slots (two chunks in flight), 128-byte swizzle
+    case 4: return run_ke_gemm_pipe<tl::RowMajor<2, 2>, float, 1, 256, 256, 512, 128, 128, 64, 32, 3, 128>(a, b, c);
+    // level 2 with two slots and ONE register step per chunk
+    case 5: return run_ke_gemm_pipe<tl::RowMajor<2, 2>, float, 2, 128, 128, 256, 64, 64, 32, 32, 2, 64>(a, b, c);
+    // level 2 with four slots, fp16 output
+    case 6: return run_ke_gemm_pipe<tl::RowMajor<2, 2>, __half, 2, 256, 256, 512, 128, 128, 64, 32, 4, 128>(a, b, c);
+    // level 2 with an odd number (3) of register steps per chunk: the register ring changes parity
+    case 7: return run_ke_gemm_pipe<tl::RowMajor<1, 2>, float, 2, 128, 128, 384, 64, 64, 96, 32, 3, 64>(a, b, c);
+    // level 2, 8 wavefronts, 16 chunks
+    case 8: return run_ke_gemm_pipe<tl::RowMajor<2, 4>, float, 2, 512, 256, 1024, 128, 256, 64, 32, 3, 128>(a, b, c);
+    default: return -1;
+  }
+}
+TT_API void tt_ke_gemm_pipe_shape(int variant, int* m, int* n, int* k, int* c_is_half) {
+  const int* t = kPipeShapes[variant];
+  *m = t[0]; *n = t[1]; *k = t[2]; *c_is_half = t[3];
+}
+
+// ---- 9. Pipeline on its own: a [kRows, kCols] tile goes chunk by chunk through a ring of
+//         kStages LDS slots (asynchronous copies, kStages - 1 chunks in flight, wait_group<N> with
+//         the loader's exact load count) and is reassembled in a second LDS area ------------------
+template <int kStages, int kRows, int kCols, int kChunkCols, typename WarpLayout>
+__global__ void k_pipeline_roundtrip(const __half* in, __half* out, int* errors) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char buf[];
+  using Global = GlobalTile<__half, tl::RowMajor<kRows, kCols>>;
+  using GIter = GTileIterator<Global, TileShape<kRows, kChunkCols>>;
+  using Shared = SharedTile<__half, tl::RowMajor<kRows, kChunkCols>, true, 128>;
+  using Loader = GlobalToSharedLoader<Shared, WarpLayout>;
+  using Pipe = Pipeline<__half, Global, Shared, GIter, Loader, kStages, GIter::sc1>;
+  static_assert(Pipe::Iterations == GIter::sc1);
+  constexpr int kChunks = GIter::sc1, kAhead = kStages - 1, kLoads = Loader::kLoadsPerLane;
+  constexpr int kThreads = tl::get_numel<WarpLayout> * WARP_SIZE;
+  __half* ring = reinterpret_cast<__half*>(buf);
+  __half* whole = ring + kStages * Shared::kNumel;   // [kRows, kCols], plain row-major
+  Pipe pipe(in, ring);
+  int bad = 0;
+#pragma unroll
+  for (int i = 0; i < kAhead && i < kChunks; ++i) {
+    pipe.commit();
+    commit_copy_group();
+  }
+  for (int k = 0; k < kChunks; ++k) {
+    if (k + kAhead <= kChunks) wait_group<kAhead - 1, kLoads>();
+    else wait_group<0>();
+    sync_threads_keep_copies();
+    if (k + kAhead < kChunks) {
+      pipe.commit();
+      commit_copy_group();
+    }
+    const __half* slot = pipe.get_dst_ptr_by_index(k);
+    bad += slot != ring + (k % kStages) * Shared::kNumel;
+    bad += pipe.get_dst_tile_by_index(k).data() != slot;
+    if (k + kAhead < kChunks && kStages >= 2) {
+      // the chunk just committed is the newest one: get_cur_dst is its slot, get_prev_dst the
+      // slot of the chunk before it
+      bad += pipe.get_cur_dst() != ring + ((k + kAhead) % kStages) * Shared::kNumel;
+      bad += pipe.get_prev_dst() != ring + ((k + kAhead - 1) % kStages) * Shared::kNumel;
+    }
+    Shared chunk(const_cast<__half*>(slot));
+    for (int e = threadIdx.x; e < kRows * kChunkCols; e += kThreads) {
+      const int r = e / kChunkCols, c = e % kChunkCols;
+      whole[r * kCols + k * kChunkCols + c] = chunk(r, c);   // logical access: undoes the swizzle
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < kRows * kCols; e += kThreads) out[e] = whole[e];
+  if (bad) atomicAdd(errors, bad);
+}
+template <int kStages, int kRows, int kCols, int kChunkCols, typename WarpLayout>
+static int run_pipeline_roundtrip(const void* in, void* out, int* errors) {
+  auto kern = k_pipeline_roundtrip<kStages, kRows, kCols, kChunkCols, WarpLayout>;
+  const int lds = (kStages * kRows * kChunkCols + kRows * kCols) * 2;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) return -2;
+  hipLaunchKernelGGL(kern, dim3(1), dim3(tl::get_numel<WarpLayout> * WARP_SIZE), lds, 0, static_cast<const __half*>(in),
+                     static_cast<__half*>(out), errors);
+  return launch_status();
+}
+TT_API int tt_pipeline_roundtrip(int variant, const void* in, void* out, int* errors) {
+  switch (variant) {
+    case 0: return run_pipeline_roundtrip<2, 64, 256, 64, tl::RowMajor<2, 2>>(in, out, errors);
+    case 1: return run_pipeline_roundtrip<3, 64, 256, 64, tl::RowMajor<2, 2>>(in, out, errors);
+    case 2: return run_pipeline_roundtrip<3, 64, 512, 64, tl::RowMajor<1, 1>>(in, out, errors);
+    case 3: return run_pipeline_roundtrip<4, 32, 512, 64, tl::RowMajor<2, 1>>(in, out, errors);
+    default: return -1;
+  }
+}
+TT_API void tt_pipeline_shape(int variant, int* rows, int* cols) {
+  static const int t[4][2] = {{64, 256}, {64, 256}, {64, 512}, {32, 512}};
+  *rows = t[variant][0]; *cols = t[variant][1];
+}
+
+// ---- 10. a strided sub-tile as the loader's destination (the register-staged path), next to an
+//          asynchronous load of the other half of the same LDS tile --------------------------------
+__global__ void k_g2s_subtile(const __half* in, __half* out) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char buf[];
+  using WarpLayout = tl::RowMajor<2, 2>;
+  using Global = GlobalTile<__half, tl::RowMajor<64, 128>>;
+  using GIter = GTileIterator<Global, TileShape<64, 64>>;
+  using Shared = SharedTile<__half, tl::RowMajor<64, 128>, true, 128>;
+  using SIter = STileIterator<Shared, TileShape<64, 64>>;
+  using Sub = typename SIter::NewTile;
+  static_assert(!GlobalToSharedLoader<Sub, WarpLayout>::kDirectCapable, "a strided sub-tile cannot be filled LDS-direct");
+  static_assert(GlobalToSharedLoader<Shared, WarpLayout>::kDirectCapable, "a whole contiguous tile can");
+  __half* lds = reinterpret_cast<__half*>(buf);
+  for (int e = threadIdx.x; e < 64 * 128; e += 256) lds[e] = __float2half(-1.f);
+  __syncthreads();
+  Global g(in);
+  GIter gi(in);
+  Shared s(lds);
+  SIter si(lds);
+  GlobalToSharedLoader<Sub, WarpLayout> load_sub;
+  auto right = si(1);
+  load_sub(gi(1), right);           // right half only
+  __copy_async();
+  __syncthreads();
+  SharedToGlobalStorer<Shared, WarpLayout> store;
+  Global go(out);
+  store(s, go);
+}
+TT_API int tt_g2s_subtile(const void* in, void* out) {
+  hipLaunchKernelGGL(k_g2s_subtile, dim3(1), dim3(256), 64 * 128 * 2, 0, static_cast<const __half*>(in),
+                     static_cast<__half*>(out));
+  return launch_status();
+}
+
+// ---- 11. where a wavefront's share of a tile starts and how many base tiles it walks over:
+//          warp::GlobalOffsetHelper / SharedOffsetHelper / ExecCounter for the three WarpReuse
+//          modes (include/cell/copy/warp.hpp:158-300) -------------------------------------------
+template <typename WarpLayout, WarpReuse kMode, typename Tile, typename BaseShape>
+__global__ void k_warp_helpers(long long* out) {
+  using Exec = warp::ExecCounter<BaseShape, Tile, WarpLayout, kMode>;
+  const int wid = threadIdx.x / WARP_SIZE;
+  if (threadIdx.x % WARP_SIZE == 0) {
+    out[wid * 6 + 0] = warp::warp_row_id<WarpLayout>();
+    out[wid * 6 + 1] = warp::warp_col_id<WarpLayout>();
+    out[wid * 6 + 2] = warp::GlobalOffsetHelper<WarpLayout, kMode>{}.template get_warp_offset<Tile>();
+    out[wid * 6 + 3] = warp::SharedOffsetHelper<WarpLayout, BaseShape, Tile, kMode>{}.get_warp_offset();
+    out[wid * 6 + 4] = Exec::row_exec_count();
+    out[wid * 6 + 5] = Exec::col_exec_count();
+  }
+}
+struct Base16x32 { static constexpr int kRows = 16, kCols = 32; };
+struct Base32x16 { static constexpr int kRows = 32, kCols = 16; };
+template <typename WarpLayout, typename Tile, typename BaseShape>
+static int run_warp_helpers(int mode, long long* out) {
+  const dim3 block(tl::get_numel<WarpLayout> * WARP_SIZE);
+  if (mode == 0) hipLaunchKernelGGL((k_warp_helpers<WarpLayout, WarpReuse::kCont, Tile, BaseShape>), dim3(1), block, 0, 0, out);
+  else if (mode == 1) hipLaunchKernelGGL((k_warp_helpers<WarpLayout, WarpReuse::kRowReuseCont, Tile, BaseShape>), dim3(1), block, 0, 0, out);
+  else hipLaunchKernelGGL((k_warp_helpers<WarpLayout, WarpReuse::kColReuseCont, Tile, BaseShape>), dim3(1), block, 0, 0, out);
+  return launch_status();
+}
+// layout 0: RowMajor<2,2> wavefronts, row-major [128, 256] tile with row stride 512
+// layout 1: RowMajor<4,1> wavefronts, row-major [128, 64] tile
+// layout 2: ColMajor<2,2> wavefronts, column-major [128, 64] tile with column stride 256
+TT_API int tt_warp_helpers(int layout, int mode, long long* out) {
+  switch (layout) {
+    case 0: return run_warp_helpers<tl::RowMajor<2, 2>, GlobalTile<__half, tl::RowMajor<128, 256, 512>>, Base16x32>(mode, out);
+    case 1: return run_warp_helpers<tl::RowMajor<4, 1>, GlobalTile<__half, tl::RowMajor<128, 64>>, Base16x32>(mode, out);
+    case 2: return run_warp_helpers<tl::ColMajor<2, 2>, GlobalTile<__half, tl::ColMajor<128, 64, 256>>, Base32x16>(mode, out);
+    default: return -1;
+  }
+}
+
+// ---- 12. STileIterator2 over plain, block and block-swizzled layouts: the six layouts of
+//          tests/cpp/types/test_stile_iterator.cu:48-236 (print-only there) -----------------------
+template <typename Shared, typename SIter>
+__global__ void k_stile_iterator2(float* out_xy, float* out_rows, float* out_cols, float* out_single) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char buf[];
+  using DType = typename Shared::DType;
+  DType* lds = reinterpret_cast<DType*>(buf);
+  for (int i = 0; i < Shared::kNumel; ++i) lds[i] = static_cast<DType>((float)i);
+  Shared tile(lds);
+  SIter it(&tile);
+  constexpr int cr = SIter::kChunkRows, cc = SIter::kChunkCols;
+  for (int x = 0; x < SIter::sc0; ++x)
+    for (int y = 0; y < SIter::sc1; ++y) {
+      auto sub = it(x, y);
+      auto row_strip = it(x, _);
+      auto col_strip = it(_, y);
+      auto sub_r = row_strip(y);
+      auto sub_c = col_strip(x);
+      for (int r = 0; r < cr; ++r)
+        for (int c = 0; c < cc; ++c) {
+          const int o = ((x * SIter::sc1 + y) * cr + r) * cc + c;
+          out_xy[o] = to_float(sub(r, c));
+          out_rows[o] = to_float(sub_r(r, c));
+          out_cols[o] = to_float(sub_c(r, c));
+          if constexpr (SIter::sc0 == 1 || SIter::sc1 == 1) out_single[o] = to_float(it(SIter::sc0 == 1 ? y : x)(r, c));
+        }
+    }
+  // to_tile gives the parent back
+  auto parent = it.to_tile();
+  if (parent.data() != tile.data()) out_xy[0] = -1.f;
+}
+template <typename Layout, int kChunkRows, int kChunkCols>
+static int run_stile_iterator2(float* a, float* b, float* c, float* d) {
+  using Shared = SharedTile<__half, Layout>;
+  using SIter = STileIterator2<Shared, TileShape<kChunkRows, kChunkCols>>;
+  hipLaunchKernelGGL((k_stile_iterator2<Shared, SIter>), dim3(1), dim3(1), Shared::kNumel * 2, 0, a, b, c, d);
+  return launch_status();
+}
+TT_API int tt_stile_iterator2(int variant, float* out_xy, float* out_rows, float* out_cols, float* out_single) {
+  switch (variant) {
+    case 0: return run_stile_iterator2<tl::RowMajor<4, 24>, 4, 8>(out_xy, out_rows, out_cols, out_single);
+    case 1: return run_stile_iterator2<tl::ColMajor<24, 4>, 8, 4>(out_xy, out_rows, out_cols, out_single);
+    case 2: return run_stile_iterator2<tl::BlockRowMajor<tl::RowMajor<4, 16>, tl::RowMajor<2, 4>>, 4, 8>(out_xy, out_rows, out_cols, out_single);
+    case 3: return run_stile_iterator2<tl::BlockColMajor<tl::ColMajor<16, 4>, tl::ColMajor<4, 2>>, 8, 4>(out_xy, out_rows, out_cols, out_single);
+    case 4: return run_stile_iterator2<tl::BlockRowMajor<tl::RowMajor<8, 16>, SwizzledLayout<tl::RowMajor<2, 4>, Swizzle<1, 0, 2>>>, 8, 4>(out_xy, out_rows, out_cols, out_single);
+    case 5: return run_stile_iterator2<tl::BlockColMajor<tl::ColMajor<32, 8>, SwizzledLayout<tl::ColMajor<4, 4>, Swizzle<2, 0, 2>>>, 8, 8>(out_xy, out_rows, out_cols, out_single);
+    // a genuinely two-dimensional chunking (the reference leaves (x, y) unimplemented)
+    case 6: return run_stile_iterator2<tl::BlockRowMajor<tl::RowMajor<8, 16>, tl::RowMajor<2, 4>>, 4, 8>(out_xy, out_rows, out_cols, out_single);
+    case 7: return run_stile_iterator2<tl::RowMajor<8, 16>, 2, 4>(out_xy, out_rows, out_cols, out_single);
+    default: return -1;
+  }
+}
+
+// ---- 13. register-to-register copies, fixed-width vector moves and the remaining functors
+//          (include/cell/copy/register.hpp:10-41, vectorize.hpp:14-59, math_functor.hpp) ----------
+__global__ void k_reg_copy(const float* in, float* out_tile, float* out_base) {
+  using WarpLayout = tl::RowMajor<1, 1>;
+  using Global = GlobalTile<float, tl::RowMajor<32, 64>>;
+  using Reg = RegTile<BaseTileRowMajor<float>, tl::RowMajor<2, 4>>;
+  Global g(in), go(out_tile), gb(out_base);
+  Reg r, copy, only_one;
+  GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+  g2r(g, r);
+  RegTileCopy<Reg> tile_copy;
+  tile_copy(r, copy);
+  BaseTileCopy<typename Reg::DType> base_copy;
+  base_copy(r(1, 2), only_one(1, 2));   // one base tile; the rest stays zero
+  RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+  r2g(copy, go);
+  r2g(only_one, gb);
+}
+TT_API int tt_reg_copy(const void* in, void* out_tile, void* out_base) {
+  hipLaunchKernelGGL(k_reg_copy, dim3(1), dim3(64), 0, 0, static_cast<const float*>(in), static_cast<float*>(out_tile),
+                     static_cast<float*>(out_base));
+  return launch_status();
+}
+__global__ void k_vectorize(const __half* hin, __half* hout, const float* fin, float* fout) {
+  const int t = threadIdx.x;
+  Vectorize<__half, 2> h2;   // 32 bits
+  Vectorize<__half, 4> h4;   // 64 bits
+  Vectorize<__half, 8> h8;   // 128 bits
+  Vectorize<float, 2> f2;
+  Vectorize<float, 4> f4;
+  static_assert(Vectorize<__half, 8>::vectorize_bits == 128 && Vectorize<float, 2>::vectorize_bits == 64 &&
+                Vectorize<__half, 2>::vectorize_nums == 2);
+  h2(hin + 2 * t, hout + 2 * t);                      // elements [0, 128)
+  h4(hin + 128 + 4 * t, hout + 128 + 4 * t);          // [128, 384)
+  h8(hin + 384 + 8 * t, hout + 384 + 8 * t);          // [384, 896)
+  f2(fin + 2 * t, fout + 2 * t);                      // [0, 128)
+  f4.copy(fin + 128 + 4 * t, fout + 128 + 4 * t);     // [128, 384)
+}
+TT_API int tt_vectorize(const void* hin, void* hout, const void* fin, void* fout) {
+  hipLaunchKernelGGL(k_vectorize, dim3(1), dim3(64), 0, 0, static_cast<const __half*>(hin), static_cast<__half*>(hout),
+                     static_cast<const float*>(fin), static_cast<float*>(fout));
+  return launch_status();
+}
+// out_add = x + rowvec (BroadcastAdd), out_log = log(relu(x) + 1), out_min = min(x, y),
+// out_div = x / (|y| + 1), out_max = max(x, y), out_mul = rowvec * x (BroadcastMul), out_sub = x - y
+__global__ void k_functors(const float* xin, const float* yin, float* out_add, float* out_log, float* out_min,
+                           float* out_div, float* out_max, float* out_mul, float* out_sub) {
+  using WarpLayout = tl::RowMajor<2, 1>;
+  using Global = GlobalTile<float, tl::RowMajor<64, 32>>;
+  using Reg = RegTile<BaseTileRowMajor<float>, tl::RowMajor<2, 2>>;
+  using Vec = RegTile<float, tl::RowMajor<Reg::kRows, 4>>;
+  Global gx(xin), gy(yin);
+  Reg x, y, t, one;
+  GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
+  g2r(gx, x);
+  g2r(gy, y);
+  RegToGlobalStorer<Global, Reg, WarpLayout> r2g;
+  // the row vector: row sums of x
+  Vec v;
+  compute::SumReduce<Reg, tl::Layout::kRowMajor> rsum;
+  rsum(x, v);
+  { copy_tile(x, t); compute::BroadcastAdd<Vec, Reg, tl::Layout::kRowMajor> f; f(v, t); Global g(out_add); r2g(t, g); }
+  { copy_tile(x, t); compute::BroadcastMul<Vec, Reg, tl::Layout::kRowMajor> f; f(v, t); Global g(out_mul); r2g(t, g); }
+  {
+    compute::RegTileRelu<Reg> relu; relu(x, t);
+    compute::BroadcastScalar<Reg, compute::Add<float>> add1; add1(t, 1.0f, t);
+    compute::RegTileLog<Reg> lg; lg(t, t);
+    Global g(out_log); r2g(t, g);
+  }
+  { compute::RegTileMin<Reg> f; f(x, y, t); Global g(out_min); r2g(t, g); }
+  { compute::RegTileMax<Reg> f; f(x, y, t); Global g(out_max); r2g(t, g); }
+  { compute::RegTileSub<Reg> f; f(x, y, t); Global g(out_sub); r2g(t, g); }
+  {
+    compute::RegTileMul<Reg> sq; sq(y, y, one);                                   // y^2
+    compute::BroadcastScalar<Reg, compute::Add<float>> add1; add1(one, 1.0f, one);  // y^2 + 1
+    compute::RegTileDiv<Reg> f; f(x, one, t);
+    Global g(out_div); r2g(t, g);
+  }
+}
+TT_API int tt_functors(const void* x, const void* y, void* o_add, void* o_log, void* o_min, void* o_div, void* o_max,
+                       void* o_mul, void* o_sub) {
+  hipLaunchKernelGGL(k_functors, dim3(1), dim3(128), 0, 0, static_cast<const float*>(x), static_cast<const float*>(y),
+                     static_cast<float*>(o_add), static_cast<float*>(o_log), static_cast<float*>(o_min),
+                     static_cast<float*>(o_div), static_cast<float*>(o_max), static_cast<float*>(o_mul),
+                     static_cast<float*>(o_sub));
+  return launch_status();
 }

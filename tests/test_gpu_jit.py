@@ -42,7 +42,7 @@ def test_jit_vector_add():
     assert again._handle == kern._handle                          # in-process cache
 
 
-@pytest.mark.parametrize("level,stages", [(0, 1), (1, 2)])
+@pytest.mark.parametrize("level,stages", [(0, 1), (1, 2), (2, 3)])
 def test_jit_gemm_uses_the_requested_tiles(level, stages):
     from tilefusion_amd import jit
     m, n, k, tm, tn, tk = 192, 320, 160, 96, 160, 32      # 96 x 160 tiles: no ahead-of-time instance

@@ -44,6 +44,16 @@ def lib():
     lib.tt_ke_fused_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 5
     lib.tt_ke_flash.argtypes = [_i, _vp, _vp, _vp, _vp]
     lib.tt_ke_flash_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 6
+    lib.tt_ke_gemm_pipe.argtypes = [_i, _vp, _vp, _vp]
+    lib.tt_ke_gemm_pipe_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 4
+    lib.tt_pipeline_roundtrip.argtypes = [_i, _vp, _vp, _vp]
+    lib.tt_pipeline_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 2
+    lib.tt_g2s_subtile.argtypes = [_vp, _vp]
+    lib.tt_warp_helpers.argtypes = [_i, _i, _vp]
+    lib.tt_stile_iterator2.argtypes = [_i, _vp, _vp, _vp, _vp]
+    lib.tt_reg_copy.argtypes = [_vp, _vp, _vp]
+    lib.tt_vectorize.argtypes = [_vp, _vp, _vp, _vp]
+    lib.tt_functors.argtypes = [_vp] * 9
     return lib
 
 
@@ -178,3 +188,144 @@ def test_ke_flash_attention_composed_from_primitives(lib, variant):
     ref = N.attention_ref(q, kk, v, causal=bool(causal.value))
     ok, r, ab = N.check_close(o, ref)
     assert ok, (variant, r, ab)
+
+
+# ---- asynchronous copies, Pipeline and the pipelined GEMMs ----------------------------------------
+
+@pytest.mark.parametrize("variant", range(9))
+def test_ke_gemm_level1_and_level2_pipelines(lib, variant):
+    # variants 0-3 are the reference's cases 1-4 (tests/python/test_gemm.py:75-135): 64 x 64 x 64
+    # tiles, level 1 with 2 ring slots, level 2 with 3; the others vary slots (2, 3, 4), register
+    # steps per chunk (1, 2, 3), wavefront layouts and the output type
+    m, n, k, h = (_i(), _i(), _i(), _i())
+    lib.tt_ke_gemm_pipe_shape(variant, m, n, k, h)
+    a, b = oracle.make_c1_gemm_inputs(m.value, n.value, k.value, seed=500 + variant)
+    c = torch.full((m.value, n.value), float("nan"), device=DEV, dtype=torch.float16 if h.value else torch.float32)
+    assert lib.tt_ke_gemm_pipe(variant, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.data_ptr()) == 0
+    ref = N.gemm_ref(a, b)
+    assert N.rel_l2(c, ref) <= 1e-3 and N.max_abs(c, ref) <= 2e-2 * max(1.0, float(ref.abs().max()))
+    # integer operands: the products and sums are exact in fp32, so any chunk read too early or
+    # from the wrong ring slot shows as a wrong integer
+    g = torch.Generator().manual_seed(variant)
+    a = torch.randint(-2, 3, (m.value, k.value), generator=g).half()
+    b = torch.randint(-2, 3, (n.value, k.value), generator=g).half()
+    for _ in range(3):
+        c.fill_(float("nan"))
+        assert lib.tt_ke_gemm_pipe(variant, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.data_ptr()) == 0
+        assert torch.equal(c.float().cpu(), N.gemm_ref(a, b))
+
+
+@pytest.mark.parametrize("variant", range(4))
+def test_pipeline_ring_with_asynchronous_copies_is_exact(lib, variant):
+    # 2, 3, 3 and 4 ring slots; stages - 1 chunks in flight, wait_group<stages - 2> per chunk
+    r, c = _i(), _i()
+    lib.tt_pipeline_shape(variant, r, c)
+    n = r.value * c.value
+    src = ((torch.arange(n) * 3 + variant) % 2048).half().to(DEV)
+    for _ in range(3):
+        dst = torch.full((n,), -1, dtype=torch.float16, device=DEV)
+        err = torch.zeros(1, dtype=torch.int32, device=DEV)
+        assert lib.tt_pipeline_roundtrip(variant, src.data_ptr(), dst.data_ptr(), err.data_ptr()) == 0
+        assert int(err.item()) == 0          # get_dst_ptr_by_index / get_cur_dst / get_prev_dst
+        assert torch.equal(src, dst)
+
+
+def test_loader_fills_a_strided_subtile_through_registers(lib):
+    src = (torch.arange(64 * 128) % 2048).half().reshape(64, 128)
+    dst = torch.zeros(64, 128, dtype=torch.float16, device=DEV)
+    assert lib.tt_g2s_subtile(src.to(DEV).data_ptr(), dst.data_ptr()) == 0
+    want = torch.full((64, 128), -1.0, dtype=torch.float16)
+    want[:, 64:] = src[:, 64:]
+    assert torch.equal(dst.cpu(), want)
+
+
+# ---- warp helpers ------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("layout", range(3))
+@pytest.mark.parametrize("mode", range(3))
+def test_warp_offset_helpers_and_exec_counter(lib, layout, mode):
+    # (wavefront grid, its order, tile layout, base tile) of tt_warp_helpers' three layouts
+    wr, wc, wkind, tile, base = [
+        (2, 2, L.ROW_MAJOR, L.row_major(128, 256, 512), (16, 32)),
+        (4, 1, L.ROW_MAJOR, L.row_major(128, 64), (16, 32)),
+        (2, 2, L.COL_MAJOR, L.col_major(128, 64, 256), (32, 16)),
+    ][layout]
+    name = ["kCont", "kRowReuseCont", "kColReuseCont"][mode]
+    out = torch.full((wr * wc, 6), -1, dtype=torch.int64, device=DEV)
+    assert lib.tt_warp_helpers(layout, mode, out.data_ptr()) == 0
+    got = out.cpu().tolist()
+    rows, cols = L.warp_tile_shape(tile.rows, tile.cols, wr, wc, name)
+    for wid in range(wr * wc):
+        i, j = L.warp_coords(wid, wr, wc, wkind)
+        off = L.warp_global_offset(tile, wr, wc, i, j, name)
+        assert got[wid] == [i, j, off, off, rows // base[0], cols // base[1]], (wid, got[wid])
+
+
+# ---- STileIterator2 -----------------------------------------------------------------------------------
+
+def _stile2_case(variant):
+    rm, cm = L.row_major, L.col_major
+    B, S = L.BlockMatrixLayout, L.SwizzledLayout
+    return [
+        (rm(4, 24), 4, 8), (cm(24, 4), 8, 4),
+        (B(rm(4, 16), rm(2, 4)), 4, 8), (B(cm(16, 4), cm(4, 2)), 8, 4),
+        (B(rm(8, 16), S(rm(2, 4), 1, 0, 2)), 8, 4), (B(cm(32, 8), S(cm(4, 4), 2, 0, 2)), 8, 8),
+        (B(rm(8, 16), rm(2, 4)), 4, 8), (rm(8, 16), 2, 4),
+    ][variant]
+
+
+@pytest.mark.parametrize("variant", range(8))
+def test_stile_iterator2_subtiles_are_the_parents_elements(lib, variant):
+    # the buffer holds its own index, so element (r, c) of sub-tile (x, y) must read
+    # parent_layout(x * chunk_rows + r, y * chunk_cols + c); variants 0-5 are the layouts of
+    # tests/cpp/types/test_stile_iterator.cu:48-236, 6-7 chunk in both dimensions
+    layout, cr, cc = _stile2_case(variant)
+    sc0, sc1 = layout.rows // cr, layout.cols // cc
+    n = layout.rows * layout.cols
+    outs = [torch.full((n,), -7.0, device=DEV) for _ in range(4)]
+    assert lib.tt_stile_iterator2(variant, *[o.data_ptr() for o in outs]) == 0
+    want = torch.tensor([layout(x * cr + r, y * cc + c) for x in range(sc0) for y in range(sc1)
+                         for r in range(cr) for c in range(cc)], dtype=torch.float32)
+    assert sorted(want.tolist()) == list(range(n))        # the layout is a bijection
+    for o in outs[:3]:                                     # (x, y), (x, _)(y), (_, y)(x)
+        assert torch.equal(o.cpu(), want)
+    if sc0 == 1 or sc1 == 1:                               # single-index form
+        assert torch.equal(outs[3].cpu(), want)
+
+
+# ---- register copies, vector moves, remaining functors ----------------------------------------------
+
+def test_reg_tile_copy_and_base_tile_copy(lib):
+    src = torch.arange(32 * 64, dtype=torch.float32).reshape(32, 64)
+    whole = torch.full((32, 64), -1.0, device=DEV)
+    one = torch.full((32, 64), -1.0, device=DEV)
+    assert lib.tt_reg_copy(src.to(DEV).data_ptr(), whole.data_ptr(), one.data_ptr()) == 0
+    assert torch.equal(whole.cpu(), src)
+    want = torch.zeros(32, 64)
+    want[16:32, 32:48] = src[16:32, 32:48]                # base tile (1, 2) of the 2 x 4 grid
+    assert torch.equal(one.cpu(), want)
+
+
+def test_vectorize_moves_32_64_128_bits(lib):
+    h = (torch.arange(896) % 2048).half().to(DEV)
+    f = torch.arange(384, dtype=torch.float32, device=DEV)
+    ho, fo = torch.full_like(h, -1), torch.full_like(f, -1)
+    assert lib.tt_vectorize(h.data_ptr(), ho.data_ptr(), f.data_ptr(), fo.data_ptr()) == 0
+    assert torch.equal(h, ho) and torch.equal(f, fo)
+
+
+def test_remaining_broadcast_and_map_functors(lib):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((64, 32)).astype(np.float32)
+    y = rng.standard_normal((64, 32)).astype(np.float32)
+    outs = [torch.zeros(64, 32, device=DEV) for _ in range(7)]
+    xd, yd = torch.from_numpy(x).to(DEV), torch.from_numpy(y).to(DEV)
+    assert lib.tt_functors(xd.data_ptr(), yd.data_ptr(), *[o.data_ptr() for o in outs]) == 0
+    o_add, o_log, o_min, o_div, o_max, o_mul, o_sub = [o.cpu().numpy() for o in outs]
+    rs = x.sum(axis=1, keepdims=True)
+    assert np.allclose(o_add, x + rs, atol=1e-5)                        # BroadcastAdd
+    assert np.allclose(o_mul, x * rs, atol=1e-4)                        # BroadcastMul
+    assert np.allclose(o_log, np.log(np.maximum(x, 0) + 1), atol=1e-5)  # Relu, scalar Add, Log
+    assert np.array_equal(o_min, np.minimum(x, y)) and np.array_equal(o_max, np.maximum(x, y))
+    assert np.array_equal(o_sub, x - y)
+    assert np.allclose(o_div, x / (y * y + 1), rtol=1e-6, atol=1e-7)    # Mul, scalar Add, Div

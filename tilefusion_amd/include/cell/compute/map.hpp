@@ -89,6 +89,11 @@ using BaseTileLog = detail::ElementWise<RegTile, Log<scalar_of_t<RegTile>>>;
 template <typename RegTile>
 using RegTileLog = detail::ElementWise<RegTile, Log<scalar_of_t<RegTile>>>;
 
+template <typename RegTile>
+using BaseTileRelu = detail::ElementWise<RegTile, Relu<scalar_of_t<RegTile>>>;
+template <typename RegTile>
+using RegTileRelu = detail::ElementWise<RegTile, Relu<scalar_of_t<RegTile>>>;
+
 template <typename Src, typename Dst>
 using BaseTileConvert = detail::ElementWise2<Src, Dst, Convert<scalar_of_t<Src>, scalar_of_t<Dst>>>;
 template <typename Src, typename Dst>

@@ -28,11 +28,23 @@ DEVICE void ld_shared_st_global(void* global_dst, const void* shared_src) {
   ld_global_st_shared<kBytes>(global_dst, shared_src);
 }
 
-// Wavefront-wide LDS-direct load (global_load_lds_dwordx4): lane l's 16 bytes land at
-// lds_base + 16 * l, where lds_base is uniform over the wavefront and 16-byte aligned;
-// `global_src` is per lane.  No register staging; completion is tracked by vmcnt.
-DEVICE void ld_global_direct_to_shared_16B(void* lds_base, const void* global_src) {
-  __builtin_amdgcn_global_load_lds(global_src, (__attribute__((address_space(3))) void*)lds_base, 16, 0, 0);
+// Wavefront-wide asynchronous copy (global_load_lds_dwordx4): lane l's 16 bytes land at LDS byte
+// address `lds_wave_base` + 16 * l, where lds_wave_base is uniform over the wavefront and
+// `global_src` is per lane.  No register staging; completion is tracked by vmcnt only, and the
+// compiler is deliberately not told that LDS is written (it would otherwise drain the counter in
+// front of every LDS read): ordering against readers is the caller's wait_group<N>() + barrier,
+// exactly the contract of the reference's cp.async atom (include/cell/copy/copy_atom.hpp:18-48).
+DEVICE void ld_global_direct_to_shared_16B(unsigned lds_wave_base, const void* global_src) {
+  // readfirstlane: the value is uniform by contract, this makes it a scalar register by type
+  const unsigned base = __builtin_amdgcn_readfirstlane(lds_wave_base);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(global_src), "s"(base)
+               : "memory");
+}
+// LDS byte address of a pointer into LDS (what M0 takes).
+DEVICE unsigned lds_byte_address(const void* p) {
+  return (unsigned)(size_t)((__attribute__((address_space(3))) const char*)p);
 }
 
 }  // namespace tilefusion::cell::copy::atom

@@ -49,14 +49,19 @@ struct FragmentMap {
   }
 };
 
-template <typename Global, typename Reg, typename WarpLayout, WarpReuse kMode>
+// extent of the block one base tile covers in memory, in the form warp::ExecCounter takes
+template <typename BaseTile>
+struct BaseExtent {
+  static constexpr int kRows = BaseTileTraits<BaseTile>::kRows;
+  static constexpr int kCols = BaseTileTraits<BaseTile>::kCols;
+};
+
+// The register tile must be exactly the base tiles a wavefront walks over in its share.
+template <typename Tile, typename Reg, typename WarpLayout, WarpReuse kMode>
 struct GlobalRegCheck {
-  using BaseTile = typename Reg::DType;
-  using Traits = BaseTileTraits<BaseTile>;
-  static constexpr int kWarpRows = warp::warp_tile_rows<Global::kRows, tl::num_rows<WarpLayout>, kMode>();
-  static constexpr int kWarpCols = warp::warp_tile_cols<Global::kCols, tl::num_cols<WarpLayout>, kMode>();
-  static_assert(kWarpRows == Reg::kRows * Traits::kRows && kWarpCols == Reg::kCols * Traits::kCols,
-                "the register tile does not cover the wavefront's share of the global tile");
+  using Exec = warp::ExecCounter<BaseExtent<typename Reg::DType>, Tile, WarpLayout, kMode>;
+  static_assert(Exec::kRowExec == Reg::kRows && Exec::kColExec == Reg::kCols,
+                "the register tile does not cover the wavefront's share of the tile");
 };
 
 }  // namespace detail
@@ -73,10 +78,8 @@ struct GlobalToRegLoader {
   template <typename Global>
   DEVICE void operator()(const Global& src, Reg& dst) {
     [[maybe_unused]] detail::GlobalRegCheck<Global, Reg, WarpLayout, kMode> check;
-    int r0, c0;
-    warp::warp_origin<WarpLayout, kMode, Global>(r0, c0);
     const int lane = warp::lane_id();
-    const DType* base = src.data();
+    const DType* base = src.data() + warp::GlobalOffsetHelper<WarpLayout, kMode>{}.template get_warp_offset<Global>();
 #pragma unroll
     for (int i = 0; i < Reg::kRows; ++i)
 #pragma unroll
@@ -84,8 +87,8 @@ struct GlobalToRegLoader {
         DType* out = dst(i, j).mutable_data();
         int r, c;
         detail::FragmentMap<BaseTile>::coord(lane, 0, r, c);
-        r += r0 + i * Traits::kRows;
-        c += c0 + j * Traits::kCols;
+        r += i * Traits::kRows;
+        c += j * Traits::kCols;
         constexpr bool kContig = Traits::kIsOperand && ((Traits::kIsRowMajor && Global::kColStride == 1) ||
                                                         (!Traits::kIsRowMajor && Global::kRowStride == 1));
         if constexpr (kContig) {
@@ -96,8 +99,8 @@ struct GlobalToRegLoader {
           for (int e = 0; e < BaseTile::kNumel; ++e) {
             int rr, cc;
             detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
-            rr += r0 + i * Traits::kRows;
-            cc += c0 + j * Traits::kCols;
+            rr += i * Traits::kRows;
+            cc += j * Traits::kCols;
             out[e] = base[ptrdiff_t(rr) * Global::kRowStride + ptrdiff_t(cc) * Global::kColStride];
           }
         }
@@ -116,10 +119,9 @@ struct RegToGlobalStorer {
 
   DEVICE void operator()(const Reg& src, Global& dst) {
     [[maybe_unused]] detail::GlobalRegCheck<Global, Reg, WarpLayout, WarpReuse::kCont> check;
-    int r0, c0;
-    warp::warp_origin<WarpLayout, WarpReuse::kCont, Global>(r0, c0);
     const int lane = warp::lane_id();
-    DType* base = dst.mutable_data();
+    DType* base = dst.mutable_data() +
+                  warp::GlobalOffsetHelper<WarpLayout, WarpReuse::kCont>{}.template get_warp_offset<Global>();
 #pragma unroll
     for (int i = 0; i < Reg::kRows; ++i)
 #pragma unroll
@@ -129,8 +131,8 @@ struct RegToGlobalStorer {
         for (int e = 0; e < BaseTile::kNumel; ++e) {
           int rr, cc;
           detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
-          rr += r0 + i * Traits::kRows;
-          cc += c0 + j * Traits::kCols;
+          rr += i * Traits::kRows;
+          cc += j * Traits::kCols;
           base[ptrdiff_t(rr) * Global::kRowStride + ptrdiff_t(cc) * Global::kColStride] = in[e];
         }
       }

@@ -22,8 +22,8 @@ struct SharedToRegLoader {
   template <typename Shared>
   DEVICE void operator()(const Shared& src, Reg& dst) {
     [[maybe_unused]] detail::GlobalRegCheck<Shared, Reg, WarpLayout, kMode> check;
-    int r0, c0;
-    warp::warp_origin<WarpLayout, kMode, Shared>(r0, c0);
+    const int warp_off =
+        warp::SharedOffsetHelper<WarpLayout, detail::BaseExtent<BaseTile>, Shared, kMode>{}.get_warp_offset();
     const int lane = warp::lane_id();
     const DType* base = src.data();
 #pragma unroll
@@ -36,18 +36,18 @@ struct SharedToRegLoader {
         if constexpr (kContig) {
           int r, c;
           detail::FragmentMap<BaseTile>::coord(lane, 0, r, c);
-          r += r0 + i * Traits::kRows;
-          c += c0 + j * Traits::kCols;
+          r += i * Traits::kRows;
+          c += j * Traits::kCols;
           *reinterpret_cast<uint4*>(out) = *reinterpret_cast<const uint4*>(
-              base + src.fetch_physical_offset(r * Shared::kRowStride + c * Shared::kColStride));
+              base + src.fetch_physical_offset(warp_off + r * Shared::kRowStride + c * Shared::kColStride));
         } else {
 #pragma unroll
           for (int e = 0; e < BaseTile::kNumel; ++e) {
             int rr, cc;
             detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
-            rr += r0 + i * Traits::kRows;
-            cc += c0 + j * Traits::kCols;
-            out[e] = base[src.fetch_physical_offset(rr * Shared::kRowStride + cc * Shared::kColStride)];
+            rr += i * Traits::kRows;
+            cc += j * Traits::kCols;
+            out[e] = base[src.fetch_physical_offset(warp_off + rr * Shared::kRowStride + cc * Shared::kColStride)];
           }
         }
       }
@@ -65,8 +65,8 @@ struct RegToSharedStorer {
   template <typename Shared>
   DEVICE void operator()(const Reg& src, Shared& dst) {
     [[maybe_unused]] detail::GlobalRegCheck<Shared, Reg, WarpLayout, WarpReuse::kCont> check;
-    int r0, c0;
-    warp::warp_origin<WarpLayout, WarpReuse::kCont, Shared>(r0, c0);
+    const int warp_off = warp::SharedOffsetHelper<WarpLayout, detail::BaseExtent<BaseTile>, Shared,
+                                                  WarpReuse::kCont>{}.get_warp_offset();
     const int lane = warp::lane_id();
     DType* base = dst.mutable_data();
 #pragma unroll
@@ -78,9 +78,9 @@ struct RegToSharedStorer {
         for (int e = 0; e < BaseTile::kNumel; ++e) {
           int rr, cc;
           detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
-          rr += r0 + i * Traits::kRows;
-          cc += c0 + j * Traits::kCols;
-          base[dst.fetch_physical_offset(rr * Shared::kRowStride + cc * Shared::kColStride)] = in[e];
+          rr += i * Traits::kRows;
+          cc += j * Traits::kCols;
+          base[dst.fetch_physical_offset(warp_off + rr * Shared::kRowStride + cc * Shared::kColStride)] = in[e];
         }
       }
   }

@@ -2,6 +2,8 @@
 // (counterpart of include/cell/copy/warp.hpp:65-300).
 #pragma once
 
+#include <cstddef>
+
 #include "cell/copy/constants.hpp"
 #include "types/layout.hpp"
 #include "types/tile_shape.hpp"
@@ -49,7 +51,10 @@ struct ExecCounter {
   DEVICE static constexpr int col_exec_count() { return kColExec; }
 };
 
-// (row, col) of the first element of this wavefront's share of `Tile`, in elements.
+// (row, col) of the first element of this wavefront's share of `Tile`, in elements: with kCont
+// wavefront (i, j) owns block (i, j); with kRowReuseCont the wavefronts of row i share row block
+// i and start at column 0; with kColReuseCont those of column j share column block j and start
+// at row 0 (include/cell/copy/warp.hpp:20-47,206-231).
 template <typename WarpLayout, WarpReuse kMode, typename Tile>
 DEVICE void warp_origin(int& row, int& col) {
   constexpr int kRowsPerWarp = Tile::kRows / (int)tl::num_rows<WarpLayout>;
@@ -58,24 +63,33 @@ DEVICE void warp_origin(int& row, int& col) {
   col = kMode == WarpReuse::kRowReuseCont ? 0 : warp_col_id<WarpLayout>() * kColsPerWarp;
 }
 
+// Element offset of this wavefront's share inside a global tile (64-bit: a global tile may span
+// more than 2^31 elements).  Used by the global <-> register movers.
 template <typename WarpLayout_, WarpReuse kMode_>
 struct GlobalOffsetHelper {
   using WarpLayout = WarpLayout_;
   static constexpr WarpReuse kMode = kMode_;
   template <typename Tile>
-  DEVICE int get_warp_offset() {
+  DEVICE ptrdiff_t get_warp_offset() const {
     int r, c;
     warp_origin<WarpLayout, kMode, Tile>(r, c);
-    return r * Tile::kRowStride + c * Tile::kColStride;
+    return ptrdiff_t(r) * Tile::kRowStride + ptrdiff_t(c) * Tile::kColStride;
   }
 };
 
+// Logical element offset of this wavefront's share inside an LDS tile, to be passed through
+// SharedTile::fetch_physical_offset together with the in-share offset.  Used by the LDS <->
+// register movers.
 template <typename WarpLayout_, typename BaseShape_, typename Shared_, WarpReuse kMode_>
 struct SharedOffsetHelper {
-  DEVICE int get_warp_offset() {
+  using WarpLayout = WarpLayout_;
+  using BaseShape = BaseShape_;
+  using Shared = Shared_;
+  static constexpr WarpReuse kMode = kMode_;
+  DEVICE int get_warp_offset() const {
     int r, c;
-    warp_origin<WarpLayout_, kMode_, Shared_>(r, c);
-    return r * Shared_::kRowStride + c * Shared_::kColStride;
+    warp_origin<WarpLayout, kMode, Shared>(r, c);
+    return r * Shared::kRowStride + c * Shared::kColStride;
   }
 };
 

@@ -114,17 +114,21 @@ def gemm_jit(a, b, c, tile_m, tile_n, tile_k, num_stages=1, pipeline_level=0, wa
         raise ValueError("shapes must be a [M,K], b [N,K], c [M,N]")
     if m % tile_m or n % tile_n or k % tile_k:
         raise ValueError("tile sizes must divide the problem")
+    if pipeline_level > 0 and num_stages < 2:
+        raise ValueError("the pipelined kernels (pipeline_level 1 and 2) need num_stages >= 2")
     wr, wc = warp_layout
     rk = 32
     entry = {0: "ke_gemm", 1: "ke_gemm_level1_pipeline", 2: "ke_gemm_level2_pipeline"}[pipeline_level]
     name = f"gemm_kernel_{m}_{n}_{k}_{tile_m}_{tile_n}_{tile_k}_{num_stages}_{pipeline_level}_{wr}x{wc}"
     src = _PRELUDE + f"""
 using Config = KeGemmTraits<__half, float, tl::RowMajor<{wr}, {wc}>, {m}, {n}, {k}, {tile_m}, {tile_n}, {tile_k}, {rk}, {num_stages}, 64>;
-extern "C" __global__ void {name}(const __half* A, const __half* B, float* C) {{
+extern "C" __global__ __launch_bounds__({wr * wc * 64}) void {name}(const __half* A, const __half* B, float* C) {{
   {entry}<__half, float, Config>(A, B, C);
 }}
 """
-    lds = (tile_m * tile_k + tile_k * tile_n) * (2 if num_stages >= 2 else 1) * 2
+    # ke_gemm keeps at most two LDS buffers; the pipelined kernels keep num_stages ring slots
+    slots = num_stages if pipeline_level > 0 else (2 if num_stages >= 2 else 1)
+    lds = (tile_m * tile_k + tile_k * tile_n) * slots * 2
     kern = JitCompiler.get_or_compile_kernel(name, src)
     kern.launch((m // tile_m, n // tile_n), (wr * wc * 64,), (a, b, c), lds)
 
@@ -143,7 +147,7 @@ def fused_two_gemms_jit(a, b, c, d, tm=64, tn=64, tk=64, tp=64, warp_layout=(2, 
     name = f"fused_two_gemms_kernel_{m}_{n}_{k}_{p}_{tm}_{tn}_{tk}_{tp}_{wr}"
     src = _PRELUDE + f"""
 using Config = FusedTwoGemmsTraits<__half, float, tl::RowMajor<{wr}, {wc}>, {m}, {n}, {k}, {p}, {tm}, {tn}, {tk}, {tp}>;
-extern "C" __global__ void {name}(const __half* A, const __half* B, const __half* C, __half* D) {{
+extern "C" __global__ __launch_bounds__({wr * wc * 64}) void {name}(const __half* A, const __half* B, const __half* C, __half* D) {{
   ke_fused_two_gemms<__half, float, Config>(A, B, C, D);
 }}
 """
@@ -175,7 +179,7 @@ def flash_attention_jit(q, k, v_t, o, tile_length_q=64, tile_length_kv=64, tile_
 using Config = FlashAttentionTraits<__half, float, __half, TileShape<{lq}, {lkv}, {d}, {dv}>,
                                     TileShape<{tile_length_q}, {tile_length_kv}, {tk_}, {tp_}>, tl::RowMajor<{wr}, {wc}>,
                                     {scale!r}, {str(bool(causal)).lower()}>;
-extern "C" __global__ void {name}(const __half* Q, const __half* K, const __half* V, __half* O) {{
+extern "C" __global__ __launch_bounds__({wr * wc * 64}) void {name}(const __half* Q, const __half* K, const __half* V, __half* O) {{
   ke_flash_attention<__half, float, __half, Config>(Q, K, V, O);
 }}
 """
