@@ -31,6 +31,9 @@ typedef enum {
   TF_ERR_HIP = 4          /* a HIP runtime call failed; message holds hipGetErrorString */
 } tf_status_t;
 
+/* Element types of the dtype-generic entry points (the codes tf_scatter_nd takes as well). */
+typedef enum { TF_DTYPE_F32 = 0, TF_DTYPE_F16 = 1, TF_DTYPE_BF16 = 2 } tf_dtype_t;
+
 /* C[M,N] = A[M,K] * B[K,N], fp16 inputs, fp32 accumulate.
  * A is row-major [M,K]; B is column-major K x N, i.e. a row-major [N,K] buffer; C is
  * row-major [M,N], fp32 when c_is_f16 == 0 (the reference op) or fp16 otherwise (the
@@ -44,6 +47,17 @@ TF_API int tf_gemm_f16(const void* A, const void* B, void* C, int c_is_f16, int6
                        int64_t N, int64_t K, int tm, int tn, int tk, int num_stages,
                        int pipeline_level, void* stream);
 
+/* The same for fp16 or bf16 inputs (dtype = TF_DTYPE_F16 / TF_DTYPE_BF16, the reference's declared
+ * type set, include/kernels/dispatch_macros.hpp:6-23 and include/cell/compute/gemm.hpp:107-150):
+ * C is fp32 when c_is_f32 != 0, else of the input type.  fp16 is tf_gemm_f16.  bf16 runs the same
+ * ring kernel with v_mfma_f32_16x16x32_bf16 when M, N are multiples of 128 and K of 64; other
+ * bf16 shapes (M, N multiples of 16, K of 32) are compiled at run time from the header kernel
+ * with the caller's tile sizes (first call per shape: seconds, then cached in the process and on
+ * disk). */
+TF_API int tf_gemm(const void* A, const void* B, void* C, int dtype, int c_is_f32, int64_t M,
+                   int64_t N, int64_t K, int tm, int tn, int tk, int num_stages,
+                   int pipeline_level, void* stream);
+
 /* D[M,P] = (A[M,K] * B[K,N]) * C[N,P]; fp16 in/out, fp32 accumulate, A*B rounded to fp16
  * in registers and never written to memory.  A row-major [M,K]; B a row-major [N,K]
  * buffer; C a row-major [P,N] buffer; D row-major [M,P].  `batch` independent problems are
@@ -55,13 +69,25 @@ TF_API int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, v
                                   int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P,
                                   int tm, int tn, int tk, int tp, void* stream);
 
+/* The same for fp16 or bf16 (dtype as in tf_gemm); bf16 is compiled at run time from the header
+ * kernel (M multiple of 16, N and K of 32, P of 16). */
+TF_API int tf_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype,
+                              int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P, int tm,
+                              int tn, int tk, int tp, void* stream);
+
 /* O = softmax(scale * Q K^T (+ causal mask)) V for `batch` independent (batch x head)
  * slices laid out back to back.  fp16 in/out, fp32 scores, fp32 running max / sum.
  * Q [batch, Lq, D]; K [batch, Lkv, D]; V [batch, Lkv, Dv] when v_is_transposed == 0, or
  * [batch, Dv, Lkv] when 1 (what the reference op receives, python/ops/flash_attention.py:74);
  * O [batch, Lq, Dv].  Causal mask: key index > query index is masked
- * (include/cell/mask.hpp:75-82).  (D, Dv) must be (128, 128) or (64, 64); any Lq and Lkv
- * (a transposed V needs Lkv % 8 == 0 to keep its rows 16-byte aligned).
+ * (include/cell/mask.hpp:75-82).  (D, Dv) = (128, 128) and (64, 64) run the tuned kernels: any Lq
+ * and Lkv (a transposed V needs Lkv % 8 == 0 to keep its rows 16-byte aligned).  Other head
+ * dimensions are compiled at run time from the header kernel with the caller's tile sizes, as
+ * the reference does for every call (src/kernels/flash_attn.cu:16-55): that path needs a
+ * transposed V, D % 32 == 0, Dv % 16 == 0, Lq % 16 == 0 and Lkv % 32 == 0, else
+ * TF_ERR_UNSUPPORTED (the torch op pads and transposes so that it never fails).
+ * The tuned kernels fold softmax_scale * log2(e) into an fp16 copy of Q: exact to the stated
+ * tolerance whenever |Q| * softmax_scale * 1.4427 stays far below 65504 (saturates beyond).
  * Replaces: tilefusion::kernels::flash_attention, src/kernels/flash_attn.cu:58-152
  * (schema include/kernels/kernel_list.hpp:25-30). */
 TF_API int tf_flash_attention_fwd_f16(const void* Q, const void* K, const void* V, void* O,
@@ -69,6 +95,13 @@ TF_API int tf_flash_attention_fwd_f16(const void* Q, const void* K, const void* 
                                       int64_t Dv, int v_is_transposed, int tile_length_q,
                                       int tile_length_kv, int tile_hidden_qk, int tile_hidden_v,
                                       double softmax_scale, int causal, void* stream);
+
+/* The same for fp16 or bf16 (dtype as in tf_gemm); bf16 always takes the run-time compiled path. */
+TF_API int tf_flash_attention_fwd(const void* Q, const void* K, const void* V, void* O, int dtype,
+                                  int64_t batch, int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv,
+                                  int v_is_transposed, int tile_length_q, int tile_length_kv,
+                                  int tile_hidden_qk, int tile_hidden_v, double softmax_scale,
+                                  int causal, void* stream);
 
 /* Single-query (decoding) attention with the KV range split into `num_splits` chunks:
  * kernel 1 writes per-split partial (o, max, sum) in fp32 into `workspace`, kernel 2 merges

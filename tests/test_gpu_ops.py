@@ -95,3 +95,98 @@ def test_ops_run_on_the_current_stream():
 def test_smoke_entry():
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+# ---- shapes and element types without a tuned kernel: never an error for a legal call ---------------
+# bf16 tolerance: the oracle consumes the bf16-rounded inputs in fp32; products are accumulated in
+# fp32; what remains is the bf16 rounding (8 mantissa bits, 2^-9 relative) of the intermediate
+# (fused: A*B, attention: the softmax weights) and of the output: rel-L2 <= 4e-3, max-abs <= 4e-2.
+
+def _close_bf16(out, ref):
+    return N.rel_l2(out, ref) <= 4e-3 and N.max_abs(out, ref) <= 4e-2 * max(1.0, float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("d,dv,lq,lkv,causal", [(64, 128, 128, 256, False), (96, 96, 128, 128, True),
+                                                (48, 80, 64, 128, False), (128, 64, 40, 64, True)])
+def test_flash_attention_ops_for_head_dims_without_a_tuned_kernel(d, dv, lq, lkv, causal):
+    # (64, 128), (96, 96): run-time compiled from the header kernel as they are; (48, 80): zero-padded
+    # to (64, 80); Lq = 40: padded to 48 query rows.  Both op forms (natural and transposed V).
+    from tilefusion_amd.ops import flash_attention
+    g = torch.Generator().manual_seed(d * 1000 + dv)
+    q = torch.randn(2, lq, d, generator=g).half()
+    k = torch.randn(2, lkv, d, generator=g).half()
+    v = torch.randn(2, lkv, dv, generator=g).half()
+    scale = 1.0 / math.sqrt(d)
+    ref = N.attention_ref(q, k, v, scale, causal)
+    o = flash_attention(q.to(DEV), k.transpose(1, 2).contiguous().to(DEV), v.to(DEV), 8, 32, d, dv, scale, causal)
+    assert o.shape == (2, lq, dv)
+    ok, r, m = N.check_close(o, ref)
+    assert ok, (r, m)
+    o2 = torch.full((2, lq, dv), float("nan"), dtype=torch.float16, device=DEV)
+    torch.ops.tilefusion.flash_attention(q.to(DEV), k.to(DEV), v.transpose(1, 2).contiguous().to(DEV), o2,
+                                         8, 32, d, dv, scale, causal)
+    ok, r, m = N.check_close(o2, ref)
+    assert ok, (r, m)
+
+
+def test_flash_attention_key_length_that_cannot_be_padded_is_a_clear_error():
+    q = torch.randn(16, 96, dtype=torch.float16, device=DEV)
+    k = torch.randn(48, 96, dtype=torch.float16, device=DEV)
+    v = torch.randn(48, 96, dtype=torch.float16, device=DEV)
+    o = torch.zeros(16, 96, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="multiple of 32"):
+        torch.ops.tilefusion.flash_attention_fwd(q, k, v, o, 0.1, False)
+
+
+@pytest.mark.parametrize("m,n,k,p", [(128, 64, 48, 64), (64, 48, 64, 32), (96, 80, 112, 48), (256, 128, 64, 72)])
+def test_fused_two_gemms_op_pads_what_the_kernels_cannot_tile(m, n, k, p):
+    # K = 48, N = 48 ...: legal for the reference's 16-wide base tiles, not whole 32-deep MFMAs
+    from tilefusion_amd.ops import fused_two_gemms
+    a, b, c = oracle.make_c3_fused_inputs(m, n, k, p)
+    d = torch.full((m, p), float("nan"), device=DEV, dtype=torch.float16)
+    fused_two_gemms(a.to(DEV), b.to(DEV), c.to(DEV), d, 16, 16, 16, 8)
+    ok, r, mx = N.check_close(d, N.fused_two_gemms_ref(a, b, c))
+    assert ok, (r, mx)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (4096, 512, 256), (96, 160, 64), (128, 128, 96)])
+def test_gemm_op_bf16(m, n, k):
+    # the first two shapes run the ring kernel with the bf16 MFMA, the others the run-time compiled one
+    from tilefusion_amd.ops import gemm
+    a, b = oracle.make_c1_gemm_inputs(m, n, k, seed=77)
+    a, b = a.bfloat16(), b.bfloat16()
+    ref = N.gemm_ref(a, b)
+    c32 = torch.full((m, n), float("nan"), device=DEV)
+    gemm(a.to(DEV), b.to(DEV), c32, 32, 32, 32, 2, 1)
+    assert N.rel_l2(c32, ref) <= 1e-5, N.rel_l2(c32, ref)
+    c16 = torch.full((m, n), float("nan"), device=DEV, dtype=torch.bfloat16)
+    gemm(a.to(DEV), b.to(DEV), c16, 32, 32, 32, 3, 2)
+    assert _close_bf16(c16, ref), (N.rel_l2(c16, ref), N.max_abs(c16, ref))
+    # integer operands: exact
+    g = torch.Generator().manual_seed(3)
+    ai = torch.randint(-3, 4, (m, k), generator=g).bfloat16()
+    bi = torch.randint(-3, 4, (n, k), generator=g).bfloat16()
+    gemm(ai.to(DEV), bi.to(DEV), c32, 32, 32, 32, 1, 0)
+    assert torch.equal(c32.cpu(), N.gemm_ref(ai, bi))
+    with pytest.raises(RuntimeError, match="same dtype"):
+        gemm(a.to(DEV), b.half().to(DEV), c32, 32, 32, 32, 1, 0)
+
+
+def test_fused_two_gemms_and_flash_attention_ops_bf16():
+    from tilefusion_amd.ops import flash_attention, fused_two_gemms
+    a, b, c = [t.bfloat16() for t in oracle.make_c3_fused_inputs(256, 128, 64, 64)]
+    d = torch.full((256, 64), float("nan"), device=DEV, dtype=torch.bfloat16)
+    fused_two_gemms(a.to(DEV), b.to(DEV), c.to(DEV), d)
+    ref = N.fused_two_gemms_ref(a, b, c)
+    assert _close_bf16(d, ref), (N.rel_l2(d, ref), N.max_abs(d, ref))
+    with pytest.raises(TypeError):
+        fused_two_gemms(a.to(DEV), b.half().to(DEV), c.to(DEV), d)
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(128, 128, generator=g).bfloat16()
+    k = torch.randn(256, 128, generator=g).bfloat16()
+    v = torch.randn(256, 128, generator=g).bfloat16()
+    for causal in (False, True):
+        o = flash_attention(q.to(DEV), k.t().contiguous().to(DEV), v.to(DEV), 64, 64, 128, 128, 1 / math.sqrt(128), causal)
+        assert o.dtype == torch.bfloat16
+        ref = N.attention_ref(q, k, v, 1 / math.sqrt(128), causal)
+        assert _close_bf16(o, ref), (causal, N.rel_l2(o, ref), N.max_abs(o, ref))

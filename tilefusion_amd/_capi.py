@@ -11,6 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtilefusion_hip.so")
 
 TF_OK, TF_ERR_INVALID_ARG, TF_ERR_UNSUPPORTED, TF_ERR_LDS, TF_ERR_HIP = range(5)
+TF_DTYPE_F32, TF_DTYPE_F16, TF_DTYPE_BF16 = range(3)
 
 _vp, _i, _i64, _d, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_double, ctypes.c_size_t
 
@@ -19,6 +20,9 @@ SIGNATURES = {
     "tf_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i64, _i64, _i64, _i, _i, _i, _i, _i, _vp]),
     "tf_fused_two_gemms_f16": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _vp]),
     "tf_flash_attention_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _i, _d, _i, _vp]),
+    "tf_gemm": (_i, [_vp, _vp, _vp, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _i, _vp]),
+    "tf_fused_two_gemms": (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _vp]),
+    "tf_flash_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _i, _d, _i, _vp]),
     "tf_flash_decode_workspace_bytes": (_sz, [_i64, _i64, _i]),
     "tf_flash_decode_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i, _d, _vp]),
     "tf_flash_decode_static_max_partials": (_sz, []),

@@ -14,6 +14,7 @@
 namespace tfk {
 
 using half_t = _Float16;
+using bf16_t = __bf16;
 using half2_t = _Float16 __attribute__((ext_vector_type(2)));
 using half4_t = _Float16 __attribute__((ext_vector_type(4)));
 using half8_t = _Float16 __attribute__((ext_vector_type(8)));

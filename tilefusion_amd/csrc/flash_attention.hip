@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "jit_ops.hpp"
 
 namespace tfk {
 namespace {
@@ -603,6 +604,42 @@ int pick(const void* Q, const void* K, const void* V, void* O, int batch, int Lq
 }  // namespace
 }  // namespace tfk
 
+namespace tfk {
+namespace {
+int check_attention_args(const char* who, const void* Q, const void* K, const void* V, const void* O, int64_t batch,
+                         int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int tile_length_q, int tile_length_kv,
+                         int tile_hidden_qk, int tile_hidden_v, double softmax_scale) {
+  TFK_REQUIRE(Q && K && V && O, TF_ERR_INVALID_ARG, "%s: null pointer", who);
+  TFK_REQUIRE(batch > 0 && Lq > 0 && Lkv > 0 && D > 0 && Dv > 0, TF_ERR_INVALID_ARG, "%s: sizes must be positive", who);
+  TFK_REQUIRE(batch < 65536 && Lq < (1 << 21) && Lkv < (1 << 24), TF_ERR_INVALID_ARG, "%s: dimension too large", who);
+  TFK_REQUIRE(tile_length_q > 0 && tile_length_kv > 0 && tile_hidden_qk > 0 && tile_hidden_v > 0,
+              TF_ERR_INVALID_ARG, "%s: tile sizes must be positive", who);
+  TFK_REQUIRE(Lq % tile_length_q == 0 && Lkv % tile_length_kv == 0 && D % tile_hidden_qk == 0 &&
+                  Dv % tile_hidden_v == 0,
+              TF_ERR_INVALID_ARG, "%s: tile [%d,%d,%d,%d] does not divide problem [%lld,%lld,%lld,%lld]", who,
+              tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v, (long long)Lq,
+              (long long)Lkv, (long long)D, (long long)Dv);
+  TFK_REQUIRE(softmax_scale == softmax_scale && softmax_scale - softmax_scale == 0.0,
+              TF_ERR_INVALID_ARG, "%s: softmax_scale must be finite", who);
+  return TF_OK;
+}
+
+// Head dimensions without a tuned kernel go to a run-time instantiation of the header kernel
+// (any D %% 32 == 0, Dv %% 16 == 0 with V transposed, Lq %% 16 == 0, Lkv %% 32 == 0).
+int attention_fallback(const char* who, const void* Q, const void* K, const void* V, void* O, int dtype,
+                       int64_t batch, int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int v_is_transposed,
+                       int tq, int tkv, int thqk, int thv, double softmax_scale, int causal, hipStream_t st) {
+  TFK_REQUIRE(jit_flash_attention_supports(Lq, Lkv, D, Dv, v_is_transposed), TF_ERR_UNSUPPORTED,
+              "%s: no tuned kernel for head dims (D=%lld, Dv=%lld) (fp16 has 128/128 and 64/64), and the run-time "
+              "compiled kernel needs a transposed V, D %% 32 == 0, Dv %% 16 == 0, Lq %% 16 == 0, Lkv %% 32 == 0 "
+              "(got Lq=%lld Lkv=%lld, V %s); the torch op pads and transposes as needed",
+              who, (long long)D, (long long)Dv, (long long)Lq, (long long)Lkv,
+              v_is_transposed ? "transposed" : "in natural layout");
+  return jit_flash_attention(Q, K, V, O, dtype, batch, Lq, Lkv, D, Dv, tq, tkv, thqk, thv, softmax_scale, causal, st);
+}
+}  // namespace
+}  // namespace tfk
+
 extern "C" int tf_flash_attention_fwd_f16(const void* Q, const void* K, const void* V, void* O,
                                           int64_t batch, int64_t Lq, int64_t Lkv, int64_t D,
                                           int64_t Dv, int v_is_transposed, int tile_length_q,
@@ -610,31 +647,39 @@ extern "C" int tf_flash_attention_fwd_f16(const void* Q, const void* K, const vo
                                           int tile_hidden_v, double softmax_scale, int causal,
                                           void* stream) {
   using namespace tfk;
-  TFK_REQUIRE(Q && K && V && O, TF_ERR_INVALID_ARG, "tf_flash_attention_fwd_f16: null pointer");
-  TFK_REQUIRE(batch > 0 && Lq > 0 && Lkv > 0 && D > 0 && Dv > 0, TF_ERR_INVALID_ARG,
-              "tf_flash_attention_fwd_f16: sizes must be positive");
-  TFK_REQUIRE(batch < 65536 && Lq < (1 << 21) && Lkv < (1 << 24), TF_ERR_INVALID_ARG,
-              "tf_flash_attention_fwd_f16: dimension too large");
-  TFK_REQUIRE(tile_length_q > 0 && tile_length_kv > 0 && tile_hidden_qk > 0 && tile_hidden_v > 0,
-              TF_ERR_INVALID_ARG, "tf_flash_attention_fwd_f16: tile sizes must be positive");
-  TFK_REQUIRE(Lq % tile_length_q == 0 && Lkv % tile_length_kv == 0 && D % tile_hidden_qk == 0 &&
-                  Dv % tile_hidden_v == 0,
-              TF_ERR_INVALID_ARG,
-              "tf_flash_attention_fwd_f16: tile [%d,%d,%d,%d] does not divide problem [%lld,%lld,%lld,%lld]",
-              tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v, (long long)Lq,
-              (long long)Lkv, (long long)D, (long long)Dv);
-  TFK_REQUIRE(softmax_scale == softmax_scale && softmax_scale - softmax_scale == 0.0,
-              TF_ERR_INVALID_ARG, "tf_flash_attention_fwd_f16: softmax_scale must be finite");
-  TFK_REQUIRE((D == 128 && Dv == 128) || (D == 64 && Dv == 64), TF_ERR_UNSUPPORTED,
-              "tf_flash_attention_fwd_f16: head dims (D=%lld, Dv=%lld) must be 128/128 or 64/64",
-              (long long)D, (long long)Dv);
+  if (int rc = check_attention_args("tf_flash_attention_fwd_f16", Q, K, V, O, batch, Lq, Lkv, D, Dv, tile_length_q,
+                                    tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale))
+    return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool tuned = (D == 128 && Dv == 128) || (D == 64 && Dv == 64);
+  if (!tuned)
+    return attention_fallback("tf_flash_attention_fwd_f16", Q, K, V, O, TF_DTYPE_F16, batch, Lq, Lkv, D, Dv,
+                              v_is_transposed, tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v,
+                              softmax_scale, causal, st);
   TFK_REQUIRE(!v_is_transposed || Lkv % 8 == 0, TF_ERR_UNSUPPORTED,
               "tf_flash_attention_fwd_f16: transposed V needs Lkv %% 8 == 0");
   const float scale_log2 = (float)(softmax_scale * 1.4426950408889634);
-  hipStream_t st = static_cast<hipStream_t>(stream);
   if (D == 128)
     return pick<128, 128>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
                           v_is_transposed != 0, causal != 0, st);
   return pick<64, 64>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
                       v_is_transposed != 0, causal != 0, st);
+}
+
+extern "C" int tf_flash_attention_fwd(const void* Q, const void* K, const void* V, void* O, int dtype, int64_t batch,
+                                      int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int v_is_transposed,
+                                      int tile_length_q, int tile_length_kv, int tile_hidden_qk, int tile_hidden_v,
+                                      double softmax_scale, int causal, void* stream) {
+  using namespace tfk;
+  if (dtype == TF_DTYPE_F16)
+    return tf_flash_attention_fwd_f16(Q, K, V, O, batch, Lq, Lkv, D, Dv, v_is_transposed, tile_length_q, tile_length_kv,
+                                      tile_hidden_qk, tile_hidden_v, softmax_scale, causal, stream);
+  TFK_REQUIRE(dtype == TF_DTYPE_BF16, TF_ERR_UNSUPPORTED,
+              "tf_flash_attention_fwd: dtype must be TF_DTYPE_F16 or TF_DTYPE_BF16");
+  if (int rc = check_attention_args("tf_flash_attention_fwd", Q, K, V, O, batch, Lq, Lkv, D, Dv, tile_length_q,
+                                    tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale))
+    return rc;
+  return attention_fallback("tf_flash_attention_fwd", Q, K, V, O, dtype, batch, Lq, Lkv, D, Dv, v_is_transposed,
+                            tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale, causal,
+                            static_cast<hipStream_t>(stream));
 }

@@ -15,6 +15,7 @@
 //     straight from global memory into registers;
 //   * D is staged through LDS so that global stores are 16 bytes per lane along rows.
 #include "common.hpp"
+#include "jit_ops.hpp"
 
 namespace tfk {
 namespace {
@@ -370,23 +371,31 @@ int pick_tp(const void* A, const void* B, const void* C, void* D, int batch, int
 }  // namespace
 }  // namespace tfk
 
+namespace tfk {
+namespace {
+int check_fused_args(const char* who, const void* A, const void* B, const void* C, const void* D, int64_t batch,
+                     int64_t M, int64_t N, int64_t K, int64_t P, int tm, int tn, int tk, int tp) {
+  TFK_REQUIRE(A && B && C && D, TF_ERR_INVALID_ARG, "%s: null pointer", who);
+  TFK_REQUIRE(batch > 0 && M > 0 && N > 0 && K > 0 && P > 0, TF_ERR_INVALID_ARG, "%s: sizes must be positive", who);
+  TFK_REQUIRE(batch < 65536 && M < (1 << 30) && N < (1 << 24) && K < (1 << 24) && P < (1 << 24),
+              TF_ERR_INVALID_ARG, "%s: dimension too large", who);
+  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0 && tp > 0, TF_ERR_INVALID_ARG, "%s: tile sizes must be positive", who);
+  TFK_REQUIRE(M % tm == 0 && N % tn == 0 && K % tk == 0 && P % tp == 0, TF_ERR_INVALID_ARG,
+              "%s: tile [%d,%d,%d,%d] does not divide problem [%lld,%lld,%lld,%lld]", who, tm, tn, tk, tp,
+              (long long)M, (long long)N, (long long)K, (long long)P);
+  TFK_REQUIRE(K % 32 == 0 && N % 32 == 0 && P % 16 == 0, TF_ERR_UNSUPPORTED,
+              "%s: needs K %% 32 == 0, N %% 32 == 0, P %% 16 == 0 (got K=%lld N=%lld P=%lld); zero-pad K and N "
+              "(the torch op does)", who, (long long)K, (long long)N, (long long)P);
+  return TF_OK;
+}
+}  // namespace
+}  // namespace tfk
+
 extern "C" int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, void* D,
                                       int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P,
                                       int tm, int tn, int tk, int tp, void* stream) {
   using namespace tfk;
-  TFK_REQUIRE(A && B && C && D, TF_ERR_INVALID_ARG, "tf_fused_two_gemms_f16: null pointer");
-  TFK_REQUIRE(batch > 0 && M > 0 && N > 0 && K > 0 && P > 0, TF_ERR_INVALID_ARG,
-              "tf_fused_two_gemms_f16: sizes must be positive");
-  TFK_REQUIRE(batch < 65536 && M < (1 << 30) && N < (1 << 24) && K < (1 << 24) && P < (1 << 24),
-              TF_ERR_INVALID_ARG, "tf_fused_two_gemms_f16: dimension too large");
-  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0 && tp > 0, TF_ERR_INVALID_ARG,
-              "tf_fused_two_gemms_f16: tile sizes must be positive");
-  TFK_REQUIRE(M % tm == 0 && N % tn == 0 && K % tk == 0 && P % tp == 0, TF_ERR_INVALID_ARG,
-              "tf_fused_two_gemms_f16: tile [%d,%d,%d,%d] does not divide problem [%lld,%lld,%lld,%lld]",
-              tm, tn, tk, tp, (long long)M, (long long)N, (long long)K, (long long)P);
-  TFK_REQUIRE(K % 32 == 0 && N % 32 == 0 && P % 16 == 0, TF_ERR_UNSUPPORTED,
-              "tf_fused_two_gemms_f16: needs K %% 32 == 0, N %% 32 == 0, P %% 16 == 0 (got K=%lld N=%lld P=%lld)",
-              (long long)K, (long long)N, (long long)P);
+  if (int rc = check_fused_args("tf_fused_two_gemms_f16", A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // long N: stream the B / C tiles through the LDS ring (8-15% faster than the plain kernel's
   // load - wait - multiply per n-tile; both are bound by the latencies of one wavefront per SIMD)
@@ -394,4 +403,16 @@ extern "C" int tf_fused_two_gemms_f16(const void* A, const void* B, const void* 
     return launch_stream<4, 2>(A, B, C, D, (int)batch, (int)M, (int)N, st);
   if (N % 128 == 0) return pick_tp<128>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
   return pick_tp<32>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
+}
+
+extern "C" int tf_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype, int64_t batch,
+                                  int64_t M, int64_t N, int64_t K, int64_t P, int tm, int tn, int tk, int tp,
+                                  void* stream) {
+  using namespace tfk;
+  if (dtype == TF_DTYPE_F16) return tf_fused_two_gemms_f16(A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp, stream);
+  TFK_REQUIRE(dtype == TF_DTYPE_BF16, TF_ERR_UNSUPPORTED,
+              "tf_fused_two_gemms: dtype must be TF_DTYPE_F16 or TF_DTYPE_BF16");
+  if (int rc = check_fused_args("tf_fused_two_gemms", A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp)) return rc;
+  TFK_REQUIRE(jit_fused_supports(M, N, K, P), TF_ERR_UNSUPPORTED, "tf_fused_two_gemms: bf16 needs M %% 16 == 0");
+  return jit_fused_two_gemms(A, B, C, D, dtype, batch, M, N, K, P, tm, tn, tk, tp, static_cast<hipStream_t>(stream));
 }

@@ -22,6 +22,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "jit_ops.hpp"
 
 namespace tfk {
 namespace {
@@ -409,10 +410,13 @@ struct Ring64Shape {
   __host__ __device__ static constexpr int swizzle(int row, int c) { return c ^ ((row / 2) % 8); }
 };
 
-template <typename S, typename OutT>
+// InT is half_t or bf16_t: the two differ in the MFMA mnemonic and in the conversion of the
+// result, everything else moves 16-bit elements without looking at them.
+template <typename S, typename InT, typename OutT>
 __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
-    const half_t* __restrict__ A, const half_t* __restrict__ B, OutT* __restrict__ C, int M,
+    const InT* __restrict__ A, const InT* __restrict__ B, OutT* __restrict__ C, int M,
     int N, int K, int tiles_m, int tiles_n) {
+  constexpr bool kBf16 = std::is_same_v<InT, bf16_t>;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -492,7 +496,10 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     int done = 0;
 #pragma unroll
     for (int j = 0; j < S::TN; ++j) {
-      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bf[buf][j]), "v"(afx[buf][i]));
+      if constexpr (kBf16)
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bf[buf][j]), "v"(afx[buf][i]));
+      else
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(bf[buf][j]), "v"(afx[buf][i]));
       // after MFMA j: issue the next read if j is its position (reads spread evenly over the slot)
       if (done < n_reads && j == (done * S::TN) / n_reads + 1) {
         const int q = first + done;
@@ -656,12 +663,12 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     for (int i = 0; i < S::TM; ++i)
 #pragma unroll
       for (int j = 0; j < S::TN; j += 2) {
-        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+        typedef InT h2_t __attribute__((ext_vector_type(2)));
         unsigned x[2], y[2];
 #pragma unroll
         for (int d = 0; d < 2; ++d) {
-          const h2_t hx = {(half_t)acc[i][j][2 * d], (half_t)acc[i][j][2 * d + 1]};
-          const h2_t hy = {(half_t)acc[i][j + 1][2 * d], (half_t)acc[i][j + 1][2 * d + 1]};
+          const h2_t hx = {(InT)acc[i][j][2 * d], (InT)acc[i][j][2 * d + 1]};
+          const h2_t hy = {(InT)acc[i][j + 1][2 * d], (InT)acc[i][j + 1][2 * d + 1]};
           x[d] = __builtin_bit_cast(unsigned, hx);
           y[d] = __builtin_bit_cast(unsigned, hy);
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -692,15 +699,15 @@ using RingBig = Ring64Shape<256, 2, 2>;   // 5 units of 32 KiB
 using RingMid = Ring64Shape<128, 2, 4>;   // 9 units of 16 KiB: one workgroup per CU, requests 4 tiles ahead
 using RingMid2 = Ring64Shape<128, 2, 2>;  // 5 units of 16 KiB: two workgroups per CU cover each other's stalls
 
-template <typename S, typename OutT>
+template <typename S, typename OutT, typename InT = half_t>
 int launch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
-  auto kern = gemm_ring64_kernel<S, OutT>;
+  auto kern = gemm_ring64_kernel<S, InT, OutT>;
   constexpr int lds = S::kUnits * S::kUnitBytes;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
   TFK_LDS_OPT_IN(kern, lds);
   const int tiles_m = M / S::BM, tiles_n = N / S::BN;
   hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(S::kThreads), lds, st,
-                     static_cast<const half_t*>(A), static_cast<const half_t*>(B),
+                     static_cast<const InT*>(A), static_cast<const InT*>(B),
                      static_cast<OutT*>(C), M, N, K, tiles_m, tiles_n);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
@@ -807,23 +814,28 @@ int launch_guarded(const void* A, const void* B, void* C, int M, int N, int K, h
   return TF_OK;
 }
 
-template <typename OutT>
-int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
+bool ring64_fits(int M, int N, int K) { return M % 128 == 0 && N % 128 == 0 && K % 64 == 0; }
+
+template <typename OutT, typename InT>
+int dispatch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
   // 256 x 256 tiles do ~1.5x the work per cycle of 128 x 128 tiles (measured: 96 vs 146 us at
   // 4096^3) but come in quarters as many: compare the rounds of tiles the 256 CUs need, a round
   // of big tiles costing 4 units and a round of mid tiles 1.6.
-  if (M % 128 == 0 && N % 128 == 0 && K % 64 == 0) {
-    constexpr int64_t kCUs = 256;
-    const bool big_fits = M % 256 == 0 && N % 256 == 0;
-    const int64_t big_rounds = ((M / 256) * (N / 256) + kCUs - 1) / kCUs;
-    const int64_t mid_rounds = ((M / 128) * (N / 128) + kCUs - 1) / kCUs;
-    if (big_fits && 5 * big_rounds <= 2 * mid_rounds)
-      return launch_ring64<RingBig, OutT>(A, B, C, M, N, K, st);
-    // more 128 x 128 tiles than CUs: the 80 KiB variant, so that two workgroups share a CU
-    // (2048 x 4096 x 2048: 33.3 -> 30.5 us); otherwise the deep ring
-    if ((M / 128) * (N / 128) > kCUs) return launch_ring64<RingMid2, OutT>(A, B, C, M, N, K, st);
-    return launch_ring64<RingMid, OutT>(A, B, C, M, N, K, st);
-  }
+  constexpr int64_t kCUs = 256;
+  const bool big_fits = M % 256 == 0 && N % 256 == 0;
+  const int64_t big_rounds = ((M / 256) * (N / 256) + kCUs - 1) / kCUs;
+  const int64_t mid_rounds = ((M / 128) * (N / 128) + kCUs - 1) / kCUs;
+  if (big_fits && 5 * big_rounds <= 2 * mid_rounds)
+    return launch_ring64<RingBig, OutT, InT>(A, B, C, M, N, K, st);
+  // more 128 x 128 tiles than CUs: the 80 KiB variant, so that two workgroups share a CU
+  // (2048 x 4096 x 2048: 33.3 -> 30.5 us); otherwise the deep ring
+  if ((M / 128) * (N / 128) > kCUs) return launch_ring64<RingMid2, OutT, InT>(A, B, C, M, N, K, st);
+  return launch_ring64<RingMid, OutT, InT>(A, B, C, M, N, K, st);
+}
+
+template <typename OutT>
+int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
+  if (ring64_fits(M, N, K)) return dispatch_ring64<OutT, half_t>(A, B, C, M, N, K, st);
   if (M % 256 == 0 && N % 256 == 0 && K % ShapeBig::BK == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
     return launch_direct<ShapeBig, OutT>(A, B, C, M, N, K, st);
   if (M % 128 == 0 && N % 128 == 0 && K % 32 == 0)
@@ -834,25 +846,53 @@ int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStre
 }  // namespace
 }  // namespace tfk
 
+namespace tfk {
+namespace {
+int check_gemm_args(const char* who, const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K,
+                    int tm, int tn, int tk, int num_stages, int pipeline_level) {
+  TFK_REQUIRE(A && B && C, TF_ERR_INVALID_ARG, "%s: null pointer", who);
+  TFK_REQUIRE(M > 0 && N > 0 && K > 0, TF_ERR_INVALID_ARG, "%s: M, N, K must be positive", who);
+  TFK_REQUIRE(M < (1 << 30) && N < (1 << 30) && K < (1 << 22), TF_ERR_INVALID_ARG, "%s: dimension too large", who);
+  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0, TF_ERR_INVALID_ARG, "%s: tile sizes must be positive", who);
+  TFK_REQUIRE(M % tm == 0 && N % tn == 0 && K % tk == 0, TF_ERR_INVALID_ARG,
+              "%s: tile [%d,%d,%d] does not divide problem [%lld,%lld,%lld]", who, tm, tn, tk,
+              (long long)M, (long long)N, (long long)K);
+  TFK_REQUIRE(num_stages >= 1 && num_stages <= 3, TF_ERR_INVALID_ARG, "%s: num_stages must be 1, 2 or 3", who);
+  TFK_REQUIRE(pipeline_level >= 0 && pipeline_level <= 2, TF_ERR_INVALID_ARG,
+              "%s: pipeline_level must be 0, 1 or 2", who);
+  return TF_OK;
+}
+}  // namespace
+}  // namespace tfk
+
 extern "C" int tf_gemm_f16(const void* A, const void* B, void* C, int c_is_f16, int64_t M,
                            int64_t N, int64_t K, int tm, int tn, int tk, int num_stages,
                            int pipeline_level, void* stream) {
   using namespace tfk;
-  TFK_REQUIRE(A && B && C, TF_ERR_INVALID_ARG, "tf_gemm_f16: null pointer");
-  TFK_REQUIRE(M > 0 && N > 0 && K > 0, TF_ERR_INVALID_ARG, "tf_gemm_f16: M, N, K must be positive");
-  TFK_REQUIRE(M < (1 << 30) && N < (1 << 30) && K < (1 << 22), TF_ERR_INVALID_ARG,
-              "tf_gemm_f16: dimension too large");
+  if (int rc = check_gemm_args("tf_gemm_f16", A, B, C, M, N, K, tm, tn, tk, num_stages, pipeline_level)) return rc;
   TFK_REQUIRE(K % 8 == 0, TF_ERR_UNSUPPORTED, "tf_gemm_f16: K (%lld) must be a multiple of 8",
               (long long)K);
-  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0, TF_ERR_INVALID_ARG, "tf_gemm_f16: tile sizes must be positive");
-  TFK_REQUIRE(M % tm == 0 && N % tn == 0 && K % tk == 0, TF_ERR_INVALID_ARG,
-              "tf_gemm_f16: tile [%d,%d,%d] does not divide problem [%lld,%lld,%lld]", tm, tn, tk,
-              (long long)M, (long long)N, (long long)K);
-  TFK_REQUIRE(num_stages >= 1 && num_stages <= 3, TF_ERR_INVALID_ARG,
-              "tf_gemm_f16: num_stages must be 1, 2 or 3");
-  TFK_REQUIRE(pipeline_level >= 0 && pipeline_level <= 2, TF_ERR_INVALID_ARG,
-              "tf_gemm_f16: pipeline_level must be 0, 1 or 2");
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (c_is_f16) return dispatch<half_t>(A, B, C, (int)M, (int)N, (int)K, st);
   return dispatch<float>(A, B, C, (int)M, (int)N, (int)K, st);
+}
+
+extern "C" int tf_gemm(const void* A, const void* B, void* C, int dtype, int c_is_f32, int64_t M, int64_t N,
+                       int64_t K, int tm, int tn, int tk, int num_stages, int pipeline_level, void* stream) {
+  using namespace tfk;
+  if (dtype == TF_DTYPE_F16)
+    return tf_gemm_f16(A, B, C, c_is_f32 ? 0 : 1, M, N, K, tm, tn, tk, num_stages, pipeline_level, stream);
+  TFK_REQUIRE(dtype == TF_DTYPE_BF16, TF_ERR_UNSUPPORTED, "tf_gemm: dtype must be TF_DTYPE_F16 or TF_DTYPE_BF16");
+  if (int rc = check_gemm_args("tf_gemm", A, B, C, M, N, K, tm, tn, tk, num_stages, pipeline_level)) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  // bf16: the ring kernel where its tiles divide the problem, else a run-time instantiation of
+  // the header kernel with the caller's tiles
+  if (ring64_fits((int)M, (int)N, (int)K)) {
+    if (c_is_f32) return dispatch_ring64<float, bf16_t>(A, B, C, (int)M, (int)N, (int)K, st);
+    return dispatch_ring64<bf16_t, bf16_t>(A, B, C, (int)M, (int)N, (int)K, st);
+  }
+  TFK_REQUIRE(jit_gemm_supports(M, N, K), TF_ERR_UNSUPPORTED,
+              "tf_gemm: bf16 needs M %% 16 == 0, N %% 16 == 0, K %% 32 == 0 (got %lld, %lld, %lld)", (long long)M,
+              (long long)N, (long long)K);
+  return jit_gemm(A, B, C, dtype, c_is_f32 ? 0 : 1, M, N, K, tm, tn, tk, num_stages, pipeline_level, st);
 }

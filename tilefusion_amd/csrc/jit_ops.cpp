@@ -1,0 +1,170 @@
+// Host launchers that instantiate the header macro kernels (kernels/*_device.hpp) at run time
+// for shapes and element types the ahead-of-time kernels of this library have no instance of.
+//
+// This is the reference's own launch path (src/kernels/gemm.cu:21-59,63-142,
+// src/kernels/fused_two_gemms.cu:35-63, src/kernels/flash_attn.cu:16-55,58-152): the whole
+// problem shape and the tile sizes become template arguments of a generated wrapper, which is
+// compiled once per distinct argument set (JitCompiler caches it in the process and on disk)
+// and launched on the caller's stream.  Here it is the fallback behind the tuned entry points.
+#include <cmath>
+#include <cstring>
+#include <sstream>
+#include <string>
+
+#include "common.hpp"
+#include "jit/compiler.hpp"
+#include "jit_ops.hpp"
+
+namespace tfk {
+namespace {
+
+using tilefusion::jit::JitCompiler;
+
+const char* kPrelude =
+    "#include \"kernels/gemm_device.hpp\"\n"
+    "#include \"kernels/fused_two_gemms_device.hpp\"\n"
+    "#include \"kernels/flash_attention_device.hpp\"\n"
+    "using namespace tilefusion;\n"
+    "using namespace tilefusion::kernels;\n"
+    "namespace tl = tile_layout;\n";
+
+const char* type_name(int dtype) { return dtype == TF_DTYPE_BF16 ? "__bfloat16" : "__half"; }
+
+// A double printed so that the compiler reads back exactly the same value (hex float).
+std::string exact(double v) {
+  char buf[64];
+  snprintf(buf, sizeof(buf), "%a", v);
+  return buf;
+}
+std::string bits_of(double v) {
+  unsigned long long u;
+  memcpy(&u, &v, sizeof(u));
+  char buf[32];
+  snprintf(buf, sizeof(buf), "%016llx", u);
+  return buf;
+}
+
+int compile_and_launch(const std::string& name, const std::string& src, dim3 grid, unsigned threads,
+                       unsigned lds, void** args, hipStream_t st) {
+  TFK_REQUIRE(lds <= (unsigned)kMaxLdsBytes, TF_ERR_LDS,
+              "%s: the requested tiles need %u bytes of LDS (a CU has 160 KiB)", name.c_str(), lds);
+  hipFunction_t fn = JitCompiler::instance().get_or_compile_kernel(name, src);
+  if (!fn) {
+    set_error("%s: run-time compilation failed: %s", name.c_str(), JitCompiler::instance().last_log().c_str());
+    return TF_ERR_HIP;
+  }
+  if (lds > 64 * 1024) {
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    (void)hipGetLastError();
+  }
+  TFK_HIP_TRY(hipModuleLaunchKernel(fn, grid.x, grid.y, grid.z, threads, 1, 1, lds, st, args, nullptr));
+  return TF_OK;
+}
+
+// largest candidate that divides n (0 if none)
+int pick_divisor(int64_t n, std::initializer_list<int> candidates) {
+  for (int c : candidates)
+    if (n % c == 0) return c;
+  return 0;
+}
+
+}  // namespace
+
+bool jit_flash_attention_supports(int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int v_is_transposed) {
+  return v_is_transposed && D % 32 == 0 && Dv % 16 == 0 && Lq % 16 == 0 && Lkv % 32 == 0 && D <= 512 && Dv <= 512;
+}
+
+int jit_flash_attention(const void* Q, const void* K, const void* Vt, void* O, int dtype, int64_t batch,
+                        int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int tq, int tkv, int thqk, int thv,
+                        double scale, int causal, hipStream_t st) {
+  // The caller's tiles are used when they are whole MFMA base tiles (16 query rows per
+  // wavefront, 32-deep reductions, 16 output columns); otherwise the nearest legal ones.
+  if (tq % 16 != 0 || Lq % tq != 0 || tq > 128) tq = pick_divisor(Lq, {64, 32, 16});
+  if (tkv % 32 != 0 || Lkv % tkv != 0 || tkv > 128) tkv = pick_divisor(Lkv, {64, 32});
+  if (thqk % 32 != 0 || D % thqk != 0) thqk = (int)D;
+  if (thv % 16 != 0 || Dv % thv != 0) thv = (int)Dv;
+  TFK_REQUIRE(tq > 0 && tkv > 0, TF_ERR_UNSUPPORTED, "flash_attention: no legal tiling for Lq=%lld Lkv=%lld",
+              (long long)Lq, (long long)Lkv);
+  // wavefronts stacked along the query rows: 16 rows each, at most 4
+  int wr = tq / 16 > 4 ? 4 : tq / 16;
+  while ((tq / wr) % 16 != 0) --wr;
+  const char* T = type_name(dtype);
+  std::ostringstream name, src;
+  name << "tf_fa_" << (dtype == TF_DTYPE_BF16 ? "bf16_" : "f16_") << Lq << "_" << Lkv << "_" << D << "_" << Dv << "_"
+       << tq << "_" << tkv << "_" << thqk << "_" << thv << "_" << (causal ? 1 : 0) << "_" << wr << "_" << bits_of(scale);
+  src << kPrelude << "using Config = FlashAttentionTraits<" << T << ", float, " << T << ", TileShape<" << Lq << ", "
+      << Lkv << ", " << D << ", " << Dv << ">, TileShape<" << tq << ", " << tkv << ", " << thqk << ", " << thv
+      << ">, tl::RowMajor<" << wr << ", 1>, " << exact(scale) << ", " << (causal ? "true" : "false") << ">;\n"
+      << "extern \"C\" __global__ __launch_bounds__(" << wr * 64 << ") void " << name.str() << "(const " << T
+      << "* Q, const " << T << "* K, const " << T << "* V, " << T << "* O) {\n"
+      << "  ke_flash_attention<" << T << ", float, " << T << ", Config>(Q, K, V, O);\n}\n";
+  const unsigned lds = (unsigned)(tq * thqk + thqk * tkv + tkv * thv + tq * tkv) * 2u;
+  void* args[] = {&Q, &K, &Vt, &O};
+  return compile_and_launch(name.str(), src.str(), dim3((unsigned)(Lq / tq), (unsigned)(Dv / thv), (unsigned)batch),
+                            wr * 64, lds, args, st);
+}
+
+bool jit_gemm_supports(int64_t M, int64_t N, int64_t K) { return M % 16 == 0 && N % 16 == 0 && K % 32 == 0; }
+
+int jit_gemm(const void* A, const void* B, void* C, int dtype, int c_kind, int64_t M, int64_t N, int64_t K, int tm,
+             int tn, int tk, int num_stages, int pipeline_level, hipStream_t st) {
+  // 2 x 2 wavefronts: 32 rows and 32 columns of C per workgroup at least
+  if (tm % 32 != 0 || M % tm != 0 || tm > 128) tm = pick_divisor(M, {128, 64, 32});
+  if (tn % 32 != 0 || N % tn != 0 || tn > 128) tn = pick_divisor(N, {128, 64, 32});
+  if (tk % 32 != 0 || K % tk != 0 || tk > 128) tk = pick_divisor(K, {64, 32});
+  int wr = 2, wc = 2;
+  if (tm == 0) { tm = pick_divisor(M, {16}); wr = 1; }
+  if (tn == 0) { tn = pick_divisor(N, {16}); wc = 1; }
+  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0, TF_ERR_UNSUPPORTED, "gemm: no legal tiling for M=%lld N=%lld K=%lld",
+              (long long)M, (long long)N, (long long)K);
+  if (pipeline_level > 0 && num_stages < 2) num_stages = 2;
+  const char* T = type_name(dtype);
+  const char* CT = c_kind == 0 ? "float" : T;
+  const char* entry =
+      pipeline_level == 0 ? "ke_gemm" : (pipeline_level == 1 ? "ke_gemm_level1_pipeline" : "ke_gemm_level2_pipeline");
+  std::ostringstream name, src;
+  name << "tf_gemm_" << (dtype == TF_DTYPE_BF16 ? "bf16_" : "f16_") << (c_kind == 0 ? "f32_" : "same_") << M << "_" << N
+       << "_" << K << "_" << tm << "_" << tn << "_" << tk << "_" << num_stages << "_" << pipeline_level << "_" << wr << wc;
+  src << kPrelude << "using Config = KeGemmTraits<" << T << ", " << CT << ", tl::RowMajor<" << wr << ", " << wc << ">, " << M
+      << ", " << N << ", " << K << ", " << tm << ", " << tn << ", " << tk << ", 32, " << num_stages << ", 64>;\n"
+      << "extern \"C\" __global__ __launch_bounds__(" << wr * wc * 64 << ") void " << name.str() << "(const " << T
+      << "* A, const " << T << "* B, " << CT << "* C) {\n  " << entry << "<" << T << ", " << CT
+      << ", Config>(A, B, C);\n}\n";
+  const int slots = pipeline_level > 0 ? num_stages : (num_stages >= 2 ? 2 : 1);
+  const unsigned lds = (unsigned)(tm * tk + tk * tn) * slots * 2u;
+  void* args[] = {&A, &B, &C};
+  return compile_and_launch(name.str(), src.str(), dim3((unsigned)(M / tm), (unsigned)(N / tn)), wr * wc * 64, lds, args,
+                            st);
+}
+
+bool jit_fused_supports(int64_t M, int64_t N, int64_t K, int64_t P) {
+  return M % 16 == 0 && N % 32 == 0 && K % 32 == 0 && P % 16 == 0;
+}
+
+int jit_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype, int64_t batch, int64_t M,
+                        int64_t N, int64_t K, int64_t P, int tm, int tn, int tk, int tp, hipStream_t st) {
+  if (tm % 16 != 0 || M % tm != 0 || tm > 128) tm = pick_divisor(M, {64, 32, 16});
+  if (tn % 32 != 0 || N % tn != 0 || tn > 128) tn = pick_divisor(N, {64, 32});
+  if (tk % 32 != 0 || K % tk != 0 || tk > 128) tk = pick_divisor(K, {64, 32});
+  if (tp % 16 != 0 || P % tp != 0 || tp > 128) tp = pick_divisor(P, {64, 32, 16});
+  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0 && tp > 0, TF_ERR_UNSUPPORTED,
+              "fused_two_gemms: no legal tiling for M=%lld N=%lld K=%lld P=%lld", (long long)M, (long long)N,
+              (long long)K, (long long)P);
+  int wr = tm / 16 > 4 ? 4 : tm / 16;
+  while ((tm / wr) % 16 != 0) --wr;
+  const char* T = type_name(dtype);
+  std::ostringstream name, src;
+  name << "tf_fused_" << (dtype == TF_DTYPE_BF16 ? "bf16_" : "f16_") << M << "_" << N << "_" << K << "_" << P << "_" << tm
+       << "_" << tn << "_" << tk << "_" << tp << "_" << wr;
+  src << kPrelude << "using Config = FusedTwoGemmsTraits<" << T << ", float, tl::RowMajor<" << wr << ", 1>, " << M << ", "
+      << N << ", " << K << ", " << P << ", " << tm << ", " << tn << ", " << tk << ", " << tp << ">;\n"
+      << "extern \"C\" __global__ __launch_bounds__(" << wr * 64 << ") void " << name.str() << "(const " << T
+      << "* A, const " << T << "* B, const " << T << "* C, " << T << "* D) {\n"
+      << "  ke_fused_two_gemms<" << T << ", float, Config>(A, B, C, D);\n}\n";
+  const unsigned lds = (unsigned)(tm * tk + tk * tn + tn * tp + tm * tn) * 2u;
+  void* args[] = {&A, &B, &C, &D};
+  return compile_and_launch(name.str(), src.str(), dim3((unsigned)(M / tm), (unsigned)(P / tp), (unsigned)batch),
+                            wr * 64, lds, args, st);
+}
+
+}  // namespace tfk

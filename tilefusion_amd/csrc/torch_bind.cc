@@ -18,6 +18,13 @@
 
 #include "tilefusion_c.h"
 
+// The dtype switch of the reference (include/kernels/dispatch_macros.hpp:6-23).  This file is
+// built by the host compiler without the device headers, so the element types are ATen's.
+#define TILEFUSION_DISPATCH_HOST_TYPES
+using __half = at::Half;
+using __bfloat16 = at::BFloat16;
+#include "kernels/dispatch_macros.hpp"
+
 namespace tilefusion {
 
 #define CHECK_CUDA(x) TORCH_CHECK((x).device().is_cuda(), #x " must be a CUDA tensor.")
@@ -26,6 +33,8 @@ namespace tilefusion {
   CHECK_CUDA(x);       \
   CHECK_CONTIGUOUS(x)
 #define CHECK_HALF(x) TORCH_CHECK((x).scalar_type() == at::kHalf, #x " must be a float16 tensor.")
+#define CHECK_SAME_TYPE(x, y) \
+  TORCH_CHECK((x).scalar_type() == (y).scalar_type(), #x " and " #y " must have the same dtype.")
 
 namespace {
 
@@ -34,6 +43,26 @@ void* current_stream() { return c10::hip::getCurrentHIPStream().stream(); }
 void check_status(int status, const char* op) {
   TORCH_CHECK(status == TF_OK, "tilefusion::", op, " failed (status ", status, "): ", tf_last_error());
 }
+
+template <typename T>
+struct DtypeCode;
+template <>
+struct DtypeCode<__half> { static constexpr int value = TF_DTYPE_F16; };
+template <>
+struct DtypeCode<__bfloat16> { static constexpr int value = TF_DTYPE_BF16; };
+template <>
+struct DtypeCode<float> { static constexpr int value = TF_DTYPE_F32; };
+
+// fp16 or bf16 -> the C ABI's dtype code (fp32 operands are rejected by the caller)
+int operand_dtype(const at::Tensor& t, const char* op) {
+  int code = -1;
+  TILEFUSION_DISPATCH_ALL_TYPES(t.scalar_type(), [&] { code = DtypeCode<scalar_t>::value; });
+  TORCH_CHECK(code == TF_DTYPE_F16 || code == TF_DTYPE_BF16, "tilefusion::", op,
+              ": operands must be float16 or bfloat16 tensors.");
+  return code;
+}
+
+int64_t round_up(int64_t x, int64_t to) { return (x + to - 1) / to * to; }
 
 int64_t leading_numel(const at::Tensor& t, int64_t keep) {
   int64_t n = 1;
@@ -51,18 +80,18 @@ void gemm(const at::Tensor& A, const at::Tensor& B, at::Tensor& C, int64_t tm, i
   CHECK_INPUT(A);
   CHECK_INPUT(B);
   CHECK_INPUT(C);
-  CHECK_HALF(A);
-  CHECK_HALF(B);
-  TORCH_CHECK(C.scalar_type() == at::kFloat || C.scalar_type() == at::kHalf,
-              "C must be a float32 or float16 tensor.");
+  const int dtype = operand_dtype(A, "gemm");
+  CHECK_SAME_TYPE(A, B);
+  TORCH_CHECK(C.scalar_type() == at::kFloat || C.scalar_type() == A.scalar_type(),
+              "C must be a float32 tensor or have the dtype of A.");
   TORCH_CHECK(A.dim() == 2 && B.dim() == 2 && C.dim() == 2, "gemm expects 2-D tensors.");
   const int64_t m = A.size(0), k = A.size(1), n = B.size(0);
   TORCH_CHECK(B.size(1) == k, "B must be [N, K] (column-major K x N); got K = ", B.size(1),
               " vs ", k);
   TORCH_CHECK(C.size(0) == m && C.size(1) == n, "C must be [M, N].");
-  check_status(tf_gemm_f16(A.data_ptr(), B.data_ptr(), C.data_ptr(), C.scalar_type() == at::kHalf,
-                           m, n, k, (int)tm, (int)tn, (int)tk, (int)num_stages,
-                           (int)pipeline_level, current_stream()),
+  check_status(tf_gemm(A.data_ptr(), B.data_ptr(), C.data_ptr(), dtype, C.scalar_type() == at::kFloat,
+                       m, n, k, (int)tm, (int)tn, (int)tk, (int)num_stages, (int)pipeline_level,
+                       current_stream()),
                "gemm");
 }
 
@@ -73,10 +102,10 @@ void fused_two_gemms(const at::Tensor& A, const at::Tensor& B, const at::Tensor&
   CHECK_INPUT(B);
   CHECK_INPUT(C);
   CHECK_INPUT(D);
-  CHECK_HALF(A);
-  CHECK_HALF(B);
-  CHECK_HALF(C);
-  CHECK_HALF(D);
+  const int dtype = operand_dtype(A, "fused_two_gemms");
+  CHECK_SAME_TYPE(A, B);
+  CHECK_SAME_TYPE(A, C);
+  CHECK_SAME_TYPE(A, D);
   TORCH_CHECK(A.dim() >= 2 && A.dim() == B.dim() && A.dim() == C.dim() && A.dim() == D.dim(),
               "fused_two_gemms expects tensors of equal rank >= 2.");
   const int64_t batch = leading_numel(A, 2);
@@ -87,10 +116,33 @@ void fused_two_gemms(const at::Tensor& A, const at::Tensor& B, const at::Tensor&
   TORCH_CHECK(leading_numel(B, 2) == batch && leading_numel(C, 2) == batch &&
                   leading_numel(D, 2) == batch,
               "batch dimensions must match.");
-  check_status(tf_fused_two_gemms_f16(A.data_ptr(), B.data_ptr(), C.data_ptr(), D.data_ptr(), batch,
-                                      m, n, k, p, (int)tm, (int)tn, (int)tk, (int)tp,
-                                      current_stream()),
+  // The kernels reduce 32 values of k (and of n, in the second product) per MFMA and write 16
+  // columns per base tile.  Shapes the reference accepts with 16-wide base tiles (K or N = 48,
+  // ...) are zero-padded here: zeros add nothing to either product.  A padded P or M (bf16:
+  // 16 rows per wavefront) goes through a temporary D.
+  const int64_t kp = round_up(k, 32), np = round_up(n, 32), pp = round_up(p, 16);
+  const int64_t mp = dtype == TF_DTYPE_BF16 ? round_up(m, 16) : m;
+  if (kp == k && np == n && pp == p && mp == m) {
+    check_status(tf_fused_two_gemms(A.data_ptr(), B.data_ptr(), C.data_ptr(), D.data_ptr(), dtype, batch,
+                                    m, n, k, p, (int)tm, (int)tn, (int)tk, (int)tp, current_stream()),
+                 "fused_two_gemms");
+    return;
+  }
+  // constant_pad_nd pads from the last dimension backwards: {last_lo, last_hi, prev_lo, prev_hi}
+  at::Tensor Ap = at::constant_pad_nd(A, {0, kp - k, 0, mp - m}, 0).contiguous();
+  at::Tensor Bp = at::constant_pad_nd(B, {0, kp - k, 0, np - n}, 0).contiguous();
+  at::Tensor Cp = at::constant_pad_nd(C, {0, np - n, 0, pp - p}, 0).contiguous();
+  const bool own_d = pp != p || mp != m;
+  std::vector<int64_t> d_shape(D.sizes().begin(), D.sizes().end());
+  d_shape[d_shape.size() - 2] = mp;
+  d_shape[d_shape.size() - 1] = pp;
+  at::Tensor Dp = own_d ? at::empty(d_shape, D.options()) : D;
+  // the caller's tiles no longer divide the padded problem: whole-dimension tiles always do
+  check_status(tf_fused_two_gemms(Ap.data_ptr(), Bp.data_ptr(), Cp.data_ptr(), Dp.data_ptr(), dtype, batch,
+                                  mp, np, kp, pp, (int)(mp % tm == 0 ? tm : mp), (int)np, (int)kp, (int)pp,
+                                  current_stream()),
                "fused_two_gemms");
+  if (own_d) D.copy_(Dp.narrow(-2, 0, m).narrow(-1, 0, p));
 }
 
 namespace {
@@ -101,10 +153,10 @@ void attention_impl(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& 
   CHECK_INPUT(K);
   CHECK_INPUT(V);
   CHECK_INPUT(O);
-  CHECK_HALF(Q);
-  CHECK_HALF(K);
-  CHECK_HALF(V);
-  CHECK_HALF(O);
+  const int dtype = operand_dtype(Q, op);
+  CHECK_SAME_TYPE(Q, K);
+  CHECK_SAME_TYPE(Q, V);
+  CHECK_SAME_TYPE(Q, O);
   TORCH_CHECK(Q.dim() >= 2 && Q.dim() == K.dim() && Q.dim() == V.dim() && Q.dim() == O.dim(),
               op, " expects tensors of equal rank >= 2.");
   const int64_t batch = leading_numel(Q, 2);
@@ -117,11 +169,36 @@ void attention_impl(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& 
   TORCH_CHECK(leading_numel(K, 2) == batch && leading_numel(V, 2) == batch &&
                   leading_numel(O, 2) == batch,
               "batch dimensions must match.");
-  check_status(tf_flash_attention_fwd_f16(Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(),
-                                          batch, lq, lkv, d, dv, v_transposed ? 1 : 0, (int)tq,
-                                          (int)tkv, (int)thqk, (int)thv, softmax_scale,
-                                          causal ? 1 : 0, current_stream()),
+  const int status = tf_flash_attention_fwd(Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), dtype,
+                                            batch, lq, lkv, d, dv, v_transposed ? 1 : 0, (int)tq,
+                                            (int)tkv, (int)thqk, (int)thv, softmax_scale,
+                                            causal ? 1 : 0, current_stream());
+  if (status != TF_ERR_UNSUPPORTED) {
+    check_status(status, op);
+    return;
+  }
+  // No tuned kernel for these head dimensions / this dtype, and the run-time compiled kernel
+  // wants a transposed V and whole MFMA base tiles: transpose V, zero-pad the head dimensions
+  // (zeros change neither the scores nor the kept output columns) and the query rows (extra
+  // rows are dropped).  The key length cannot be padded without changing the softmax.
+  TORCH_CHECK(lkv % 32 == 0, "tilefusion::", op, ": head dims (", d, ", ", dv, ") with ",
+              toString(Q.scalar_type()), " need a key length that is a multiple of 32 (got ", lkv, ").");
+  const int64_t dp = round_up(d, 32), dvp = round_up(dv, 16), lqp = round_up(lq, 16);
+  at::Tensor Qp = at::constant_pad_nd(Q, {0, dp - d, 0, lqp - lq}, 0).contiguous();
+  at::Tensor Kp = at::constant_pad_nd(K, {0, dp - d}, 0).contiguous();
+  at::Tensor Vt = v_transposed ? V : V.transpose(-1, -2);
+  Vt = at::constant_pad_nd(Vt, {0, 0, 0, dvp - dv}, 0).contiguous();
+  const bool own_o = dvp != dv || lqp != lq;
+  std::vector<int64_t> o_shape(O.sizes().begin(), O.sizes().end());
+  o_shape[o_shape.size() - 2] = lqp;
+  o_shape[o_shape.size() - 1] = dvp;
+  at::Tensor Op = own_o ? at::empty(o_shape, O.options()) : O;
+  check_status(tf_flash_attention_fwd(Qp.data_ptr(), Kp.data_ptr(), Vt.data_ptr(), Op.data_ptr(), dtype, batch,
+                                      lqp, lkv, dp, dvp, 1, (int)(lqp % tq == 0 ? tq : lqp),
+                                      (int)(lkv % tkv == 0 ? tkv : lkv), (int)dp, (int)dvp, softmax_scale,
+                                      causal ? 1 : 0, current_stream()),
                op);
+  if (own_o) O.copy_(Op.narrow(-2, 0, lq).narrow(-1, 0, dv));
 }
 }  // namespace
 

@@ -1,9 +1,14 @@
 // Runtime dtype -> compile-time type switch for host launchers (counterpart of
 // include/kernels/dispatch_macros.hpp:6-23).  `TYPE` is an at::ScalarType; the body sees the
 // element type as `scalar_t` (__half / __bfloat16 / float).
+//
+// A host-only translation unit that cannot include the device headers defines
+// TILEFUSION_DISPATCH_HOST_TYPES and provides the three type names itself.
 #pragma once
 
+#ifndef TILEFUSION_DISPATCH_HOST_TYPES
 #include "types/base.hpp"
+#endif
 
 #define TILEFUSION_DISPATCH_CASE(ENUM, CTYPE, ...) \
   case ENUM: {                                     \

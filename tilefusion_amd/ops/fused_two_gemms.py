@@ -37,9 +37,12 @@ def fused_two_gemms(
         input_c: [P, N] buffer (the column-major N x P operand).
         output: [M, P] row-major, written in place.
         tm, tn, tk, tp: the reference's tile sizes; must divide M, N, K, P.
+
+    All four tensors are float16 (as in the reference) or all bfloat16.
     """
-    _validate_tensor(input_a, "input_a")
-    _validate_tensor(input_b, "input_b")
-    _validate_tensor(input_c, "input_c")
-    _validate_tensor(output, "output")
+    dtype = torch.bfloat16 if input_a.dtype == torch.bfloat16 else torch.float16
+    _validate_tensor(input_a, "input_a", dtype)
+    _validate_tensor(input_b, "input_b", dtype)
+    _validate_tensor(input_c, "input_c", dtype)
+    _validate_tensor(output, "output", dtype)
     torch.ops.tilefusion.fused_two_gemms(input_a, input_b, input_c, output, tm, tn, tk, tp)
