@@ -108,18 +108,49 @@ TFK_DEVICE void second_product(const char* sC, const float4_t* acc1, float4_t* a
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Plain kernel: one workgroup = 64 rows (4 wavefronts x 16), n-tiles of TN, k-chunks of KC.
+//
+// Per n-tile and k-chunk the order of events is chosen for latency (at the benchmark shape
+// the whole kernel is one n-tile and one k-chunk, 64 MFMAs per wavefront, so its run time is
+// the sum of one trip to memory and one short dependent chain):
+//   * A fragments are requested FIRST (they come from HBM, the tiles of B and C from the L2),
+//     then the B tile, then the C tile, all asynchronously; the first product starts as soon
+//     as A and B have landed, with the C tile still in flight;
+//   * fragment reads run one step ahead of the MFMAs across both products;
+//   * B rows are dealt to the 16-row MFMA fragments so that the fp16-rounded accumulators of
+//     the first product are the second MFMA's operand fragment for EIGHT CONSECUTIVE n
+//     (fragment nt takes rows 32*(nt/2) + 8*(i/4) + 4*(nt%2) + i%4, i = 0..15): the matching C
+//     fragment is then one 16-byte read;
+//   * the second product is computed transposed (D^T = C^T * S^T), which leaves a lane with
+//     four consecutive columns of one row of D; pairs of tiles are re-dealt with
+//     v_permlane16_swap + ds_bpermute so that four adjacent lanes store 64 contiguous bytes.
+//     No LDS staging of D, no barrier in the epilogue.
+// ------------------------------------------------------------------------------------------
+// row of the B tile that element i of 16-row fragment nt multiplies
+__host__ __device__ constexpr int b_frag_row(int nt, int i) { return 32 * (nt / 2) + 8 * (i / 4) + 4 * (nt % 2) + i % 4; }
+// XOR key of a B-tile row: the sixteen rows of a fragment get sixteen different keys
+template <int CH>
+__host__ __device__ constexpr int b_key(int row) {
+  if constexpr (CH >= 16) return ((row >> 3) & 3) << 2 | (row & 3);
+  else return (row / (16 / CH)) % CH;
+}
+
 template <int TN, int TP, int KC>
 __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
     const half_t* __restrict__ A, const half_t* __restrict__ B, const half_t* __restrict__ C,
     half_t* __restrict__ D, int M, int N, int K, int P) {
-  constexpr int kBChunks = KC / 8;   // 16-byte chunks per sB row
-  constexpr int kCChunks = TN / 8;   // per sC row
+  constexpr int kBCh = KC / 8;       // 16-byte chunks per sB row
+  constexpr int kCCh = TN / 8;       // per sC row
   constexpr int kKSteps = KC / 32;
   constexpr int kNT = TN / 16;       // 16-wide n tiles of the first GEMM
   constexpr int kPT = TP / 16;       // 16-wide p tiles of the second GEMM
+  constexpr int kSteps2 = TN / 32;
+  constexpr int kBInstr = TN * kBCh / 64, kCInstr = (TP * kCCh + 63) / 64;   // 1 KiB requests per tile
+  constexpr int kBPerWave = (kBInstr + kWaves - 1) / kWaves, kCPerWave = (kCInstr + kWaves - 1) / kWaves;
+  static_assert(TN % 32 == 0 && KC % 32 == 0 && TP % 16 == 0, "whole MFMA base tiles");
   __shared__ __attribute__((aligned(1024))) char sB[TN * KC * 2];
-  __shared__ __attribute__((aligned(1024))) char sC[TP * TN * 2 < 1024 ? 1024 : TP * TN * 2];
-  __shared__ __attribute__((aligned(16))) half_t sD[kRowsPerBlock * TP];
+  __shared__ __attribute__((aligned(1024))) char sC[kCInstr * 1024];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -134,6 +165,48 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
 
   const int a_row = min(m0 + wave * 16 + lr, M - 1);  // clamped: rows past M are never stored
   const half_t* a_ptr = A + (size_t)a_row * K + 8 * lg;
+  const unsigned sB_addr = lds_address(sB), sC_addr = lds_address(sC);
+
+  // 1 KiB request i of the B tile covers rows 64 / kBCh * i ..; lane l fills physical chunk
+  // l % kBCh of its row with the logical chunk the key maps there.  The same for C with the
+  // plain key.  Requests beyond the tile (a C tile smaller than 1 KiB) re-fetch row 0.
+  auto request_b = [&](int n0, int k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < kBPerWave; ++q) {
+      const int i = wave + kWaves * q;
+      if (kBInstr % kWaves != 0 && i >= kBInstr) break;
+      const int row = i * (64 / kBCh) + lane / kBCh;
+      const int c = (lane % kBCh) ^ b_key<kBCh>(row);
+      lds_dma_16B(B + (size_t)(n0 + row) * K + k0 + c * 8, sB_addr + i * 1024);
+    }
+  };
+  auto request_c = [&](int n0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < kCPerWave; ++q) {
+      const int i = wave + kWaves * q;
+      if (kCInstr % kWaves != 0 && i >= kCInstr) break;
+      const int row = min(i * (64 / kCCh) + lane / kCCh, TP - 1);
+      const int c = swz<kCCh>(row, lane % kCCh);
+      lds_dma_16B(C + (size_t)(p0 + row) * N + n0 + c * 8, sC_addr + i * 1024);
+    }
+  };
+  // requests of this wavefront that are still allowed in flight when B (and A) must be there
+  const int c_requests = (kCInstr % kWaves == 0 || wave < kCInstr % kWaves) ? kCPerWave : kCPerWave - 1;
+
+  auto read_b = [&](half8_t* dst, int ks) __attribute__((always_inline)) {
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) {
+      const int row = b_frag_row(nt, lr);
+      dst[nt] = *reinterpret_cast<const half8_t*>(sB + row * KC * 2 + ((ks * 4 + lg) ^ b_key<kBCh>(row)) * 16);
+    }
+  };
+  auto read_c = [&](half8_t* dst, int s2) __attribute__((always_inline)) {
+#pragma unroll
+    for (int pt = 0; pt < kPT; ++pt) {
+      const int row = pt * 16 + lr;
+      dst[pt] = *reinterpret_cast<const half8_t*>(sC + row * TN * 2 + swz<kCCh>(row, 4 * s2 + lg) * 16);
+    }
+  };
 
   float4_t acc2[kPT];
 #pragma unroll
@@ -145,35 +218,117 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
     for (int nt = 0; nt < kNT; ++nt) acc1[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     for (int k0 = 0; k0 < K; k0 += KC) {
-      __syncthreads();  // previous readers of sB / sC are done
-      tile_to_lds<TN, KC>(B + (size_t)n0 * K + k0, K, sB, wave, lane);
-      if (k0 == 0) tile_to_lds<TP, TN>(C + (size_t)p0 * N + n0, N, sC, wave, lane);
+      const bool first_chunk = k0 == 0;
+      // previous readers of sB (and, at a new n-tile, of sC) are done
+      if (n0 != 0 || k0 != 0) barrier_lds_only();
       half8_t af[kKSteps];
+      // All three kinds of request are issued from assembly, so that the compiler places no
+      // vector-memory waits of its own (it would drain everything, the C tile included, in
+      // front of the first LDS read or the first use of an A fragment).
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks)
-        af[ks] = *reinterpret_cast<const half8_t*>(a_ptr + k0 + ks * 32);
-      wait_vmem_all();
-      __syncthreads();
-      first_product<TN, KC>(sB, af, acc1, lr, lg);
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(af[ks]) : "v"(a_ptr + k0 + ks * 32) : "memory");
+      request_b(n0, k0);
+      if (first_chunk) request_c(n0);
+      // A and B have landed once at most this wavefront's C requests are outstanding (loads
+      // retire in order); the fragment registers are re-defined behind the wait so that no use
+      // of them can be scheduled in front of it.
+      if (first_chunk && c_requests == kCPerWave) {
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kCPerWave) : "memory");
+      } else if (first_chunk && kCPerWave > 1) {
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(kCPerWave > 1 ? kCPerWave - 1 : 0) : "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) asm volatile("" : "+v"(af[ks]));
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+
+      // first product, transposed: acc1[nt] += B rows (fragment nt) x A^T, reads one step ahead
+      half8_t bf[2][kNT];
+      read_b(bf[0], 0);
+#pragma unroll
+      for (int ks = 0; ks < kKSteps; ++ks) {
+        if (ks + 1 < kKSteps) read_b(bf[(ks + 1) & 1], ks + 1);
+#pragma unroll
+        for (int nt = 0; nt < kNT; ++nt) acc1[nt] = mfma_16x16x32(bf[ks & 1][nt], af[ks], acc1[nt]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    second_product<TN, TP>(sC, acc1, acc2, lr, lg);
+    // the C tile has landed for everybody
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    // second product, transposed: lane (m = lr, group lg) holds A*B[m][32*s2 + 8*lg + 0..7] in
+    // acc1[2*s2][0..3], acc1[2*s2 + 1][0..3]; acc2[pt] += C rows (p) x that
+    half8_t cf[2][kPT];
+    read_c(cf[0], 0);
+#pragma unroll
+    for (int s2 = 0; s2 < kSteps2; ++s2) {
+      if (s2 + 1 < kSteps2) read_c(cf[(s2 + 1) & 1], s2 + 1);
+      half8_t pa;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        pa[r] = (half_t)acc1[2 * s2][r];
+        pa[4 + r] = (half_t)acc1[2 * s2 + 1][r];
+      }
+#pragma unroll
+      for (int pt = 0; pt < kPT; ++pt) acc2[pt] = mfma_16x16x32(cf[s2 & 1][pt], pa, acc2[pt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 
-  // Epilogue: acc2[pt][r] = D[m0 + 16*wave + 4*lg + r][p0 + 16*pt + lr]
+  // Epilogue: acc2[pt][r] = D[m0 + 16*wave + lr][p0 + 16*pt + 4*lg + r].
+  const int d_row0 = m0 + wave * 16;
+  if constexpr (kPT % 2 == 0) {
+    // Pairs of tiles: the 16-lane groups g and g^1 trade halves (v_permlane16_swap), after which
+    // group 0/2 holds columns 0-7 / 8-15 of tile pt and group 1/3 the same of tile pt+1, 16 bytes
+    // per lane; ds_bpermute then moves the 16 bytes of (row r, segment s) to lane 4*r + s, so
+    // that a store writes 16 rows x 64 contiguous bytes with four adjacent lanes per row.
+    const int st_row = lane >> 2, st_seg = lane & 3;
+    const int src_lane = st_row + 16 * (((st_seg & 1) << 1) | (st_seg >> 1));
+    half_t* d_lane = D + (size_t)(d_row0 + st_row) * P + p0 + 8 * st_seg;
+    const bool row_ok = d_row0 + st_row < M;
+    uint4_t v[kPT / 2];
 #pragma unroll
-  for (int pt = 0; pt < kPT; ++pt)
+    for (int pt = 0; pt < kPT; pt += 2) {
+      typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+      unsigned x[2], y[2];
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      sD[(wave * 16 + 4 * lg + r) * TP + pt * 16 + lr] = (half_t)acc2[pt][r];
-  __syncthreads();
-  constexpr int kDChunks = TP / 8;
-  for (int f = tid; f < kRowsPerBlock * kDChunks; f += kThreads) {
-    const int row = f / kDChunks, c = f % kDChunks;
-    if (m0 + row < M)
-      // streaming store: D is written once and not read again here, and an ordinary store next to
-      // the operand reads costs this HBM-bound kernel 10% (6.40 -> 5.72 us at 16384 x 128^3)
-      __builtin_nontemporal_store(*reinterpret_cast<const uint4_t*>(sD + row * TP + c * 8),
-                                  reinterpret_cast<uint4_t*>(D + (size_t)(m0 + row) * P + p0 + c * 8));
+      for (int d = 0; d < 2; ++d) {
+        const h2_t hx = {(half_t)acc2[pt][2 * d], (half_t)acc2[pt][2 * d + 1]};
+        const h2_t hy = {(half_t)acc2[pt + 1][2 * d], (half_t)acc2[pt + 1][2 * d + 1]};
+        x[d] = __builtin_bit_cast(unsigned, hx);
+        y[d] = __builtin_bit_cast(unsigned, hy);
+#if defined(__HIP_DEVICE_COMPILE__)
+        auto sw = __builtin_amdgcn_permlane16_swap(x[d], y[d], false, false);
+        x[d] = sw[0];
+        y[d] = sw[1];
+#endif
+      }
+      v[pt / 2][0] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)x[0]);
+      v[pt / 2][1] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)x[1]);
+      v[pt / 2][2] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)y[0]);
+      v[pt / 2][3] = (unsigned)__builtin_amdgcn_ds_bpermute(4 * src_lane, (int)y[1]);
+    }
+    // streaming stores: D is written once and not read again here, and an ordinary store next
+    // to the operand reads costs this latency-bound kernel 10%
+    if (row_ok) {
+#pragma unroll
+      for (int pt = 0; pt < kPT; pt += 2)
+        __builtin_nontemporal_store(v[pt / 2], reinterpret_cast<uint4_t*>(d_lane + 16 * pt));
+    }
+  } else {
+    // a single 16-column tile: 8 bytes per lane
+#pragma unroll
+    for (int pt = 0; pt < kPT; ++pt) {
+      half4_t v;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] = (half_t)acc2[pt][r];
+      if (d_row0 + lr < M)
+        *reinterpret_cast<half4_t*>(D + (size_t)(d_row0 + lr) * P + p0 + 16 * pt + 4 * lg) = v;
+    }
   }
 }
 
