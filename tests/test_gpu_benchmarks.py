@@ -18,7 +18,7 @@ def test_g2s_copy_benchmark_checks_itself():
         subprocess.check_call(["make", "-C", d])
     out = subprocess.run([path], capture_output=True, text=True, timeout=100)
     assert out.returncode == 0, out.stdout + out.stderr
-    assert out.stdout.count("|ok|") == 11 and "all configurations ok" in out.stdout
+    assert out.stdout.count("|ok|") == 22 and "all configurations ok" in out.stdout
 
 
 def test_fused_two_gemms_sweep_is_correct_on_a_few_shapes():
@@ -42,4 +42,15 @@ def test_gemm_sweep_is_correct_on_the_small_shapes():
     spec.loader.exec_module(mod)
     buf = io.StringIO()
     assert mod.run(shapes=mod.SHAPES[:5], out=buf), buf.getvalue()
+    assert "MISMATCH" not in buf.getvalue()
+
+
+def test_header_kernel_gemm_table_is_correct():
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("header_kernels", os.path.join(ROOT, "benchmarks", "gemm", "header_kernels.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    buf = io.StringIO()
+    assert mod.run(out=buf), buf.getvalue()
     assert "MISMATCH" not in buf.getvalue()

@@ -161,7 +161,8 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     for (int kk = 0; kk < kKK; ++kk) {
       const half8_t raw = *reinterpret_cast<const half8_t*>(Q + (size_t)m_ld * D + kk * 32 + lg * 8);
 #pragma unroll
-      for (int t = 0; t < 8; ++t) qf[kk][qb][t] = (half_t)((float)raw[t] * scale_log2);
+      for (int t = 0; t < 8; ++t)   // saturates instead of overflowing to inf for absurd |Q * scale|
+        qf[kk][qb][t] = (half_t)__builtin_amdgcn_fmed3f((float)raw[t] * scale_log2, -65504.f, 65504.f);
     }
   }
 
