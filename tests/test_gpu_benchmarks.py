@@ -21,6 +21,20 @@ def test_g2s_copy_benchmark_checks_itself():
     assert out.stdout.count("|ok|") == 22 and "all configurations ok" in out.stdout
 
 
+def test_mfma_ceiling_probe_runs_and_stays_under_the_peak():
+    d = os.path.join(ROOT, "benchmarks", "cpp", "mfma_ceiling")
+    path = os.path.join(d, "mfma_ceiling")
+    if not os.path.exists(path):
+        subprocess.check_call(["make", "-C", d])
+    out = subprocess.run([path], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stdout + out.stderr
+    rows = [line.split("|") for line in out.stdout.splitlines() if line.startswith("|v_mfma")]
+    assert len(rows) == 2
+    for r in rows:
+        tflops, cycles = float(r[3]), float(r[5])
+        assert 500 < tflops < 2500 and 250 <= cycles < 400, out.stdout
+
+
 def test_fused_two_gemms_sweep_is_correct_on_a_few_shapes():
     import importlib.util
 
