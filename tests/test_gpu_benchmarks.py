@@ -47,6 +47,17 @@ def test_fused_two_gemms_sweep_is_correct_on_a_few_shapes():
     assert "MISMATCH" not in buf.getvalue()
 
 
+def test_fused_launch_floor_table():
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("fused_bench2", os.path.join(ROOT, "benchmarks", "fused_two_gemms", "bench.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    rows = mod.launch_floor(out=io.StringIO())
+    (_, empty), (_, cached), (_, hbm) = rows
+    assert 0.5 < empty < cached * 1.05 and cached < 20 and hbm < 20, rows
+
+
 def test_gemm_sweep_is_correct_on_the_small_shapes():
     sys.path.insert(0, os.path.join(ROOT, "benchmarks", "gemm"))
     import importlib.util
