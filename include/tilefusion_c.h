@@ -96,7 +96,9 @@ TF_API int tf_flash_attention_fwd_f16(const void* Q, const void* K, const void* 
                                       int tile_length_kv, int tile_hidden_qk, int tile_hidden_v,
                                       double softmax_scale, int causal, void* stream);
 
-/* The same for fp16 or bf16 (dtype as in tf_gemm); bf16 always takes the run-time compiled path. */
+/* The same for fp16 or bf16 (dtype as in tf_gemm).  bf16 with (D, Dv) = (128, 128) or (64, 64) runs
+ * the tuned kernels with the bf16 MFMA, bf16 softmax weights and bf16 output; other head dimensions
+ * take the run-time compiled path as above. */
 TF_API int tf_flash_attention_fwd(const void* Q, const void* K, const void* V, void* O, int dtype,
                                   int64_t batch, int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv,
                                   int v_is_transposed, int tile_length_q, int tile_length_kv,

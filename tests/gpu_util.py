@@ -44,7 +44,12 @@ def c_attention(q, k, v, causal=False, scale=None, v_transposed=False, tiles=Non
     dv = v.shape[1] if v_transposed else v.shape[2]
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     t = tiles if tiles else (lq, lkv, d, dv)
-    o = torch.full((b, lq, dv), float("nan"), device=q.device, dtype=torch.float16)
+    o = torch.full((b, lq, dv), float("nan"), device=q.device, dtype=q.dtype)
+    if q.dtype == torch.bfloat16:   # the dtype-coded entry point: tuned bf16 kernels or the run-time compiled one
+        _capi.check(lib.tf_flash_attention_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), _capi.TF_DTYPE_BF16,
+                                               b, lq, lkv, d, dv, int(v_transposed), t[0], t[1], t[2], t[3], scale,
+                                               int(causal), stream()), "tf_flash_attention_fwd")
+        return o
     _capi.check(lib.tf_flash_attention_fwd_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), b, lq, lkv,
                                                d, dv, int(v_transposed), t[0], t[1], t[2], t[3], scale, int(causal),
                                                stream()), "tf_flash_attention_fwd_f16")

@@ -130,3 +130,37 @@ def test_large_scale_and_large_q_stay_finite():
     q_huge = (torch.randn(1, 64, 128, generator=g) * 3e4).half()
     o = c_attention(q_huge.to(DEV), k[:1].to(DEV), v[:1].to(DEV), scale=8.0)
     assert torch.isfinite(o).all()
+
+
+# bf16 runs the same tuned kernels with the bf16 MFMA, bf16 softmax weights and bf16 output.  The
+# oracle consumes the bf16-rounded inputs in fp32; what is left is the rounding of the weights and
+# of the output to 8 mantissa bits: rel-L2 <= 4e-3, max-abs <= 4e-2.
+@pytest.mark.parametrize("bh,lq,lkv,d,causal,vt", [
+    (3, 256, 512, 128, False, False), (2, 384, 384, 128, True, False), (2, 200, 333, 128, False, False),
+    (2, 100, 100, 128, True, False), (2, 256, 256, 64, True, False), (3, 130, 517, 64, False, False),
+    (2, 256, 512, 128, False, True), (2, 320, 320, 64, True, True),
+])
+def test_bf16_tuned_kernels_match_the_oracle(bh, lq, lkv, d, causal, vt):
+    g = torch.Generator().manual_seed(bh * 1000 + lq + lkv + d)
+    q = torch.randn(bh, lq, d, generator=g).bfloat16()
+    k = torch.randn(bh, lkv, d, generator=g).bfloat16()
+    v = torch.randn(bh, lkv, d, generator=g).bfloat16()
+    v_dev = v.transpose(1, 2).contiguous().to(DEV) if vt else v.to(DEV)
+    o = c_attention(q.to(DEV), k.to(DEV), v_dev, causal=causal, v_transposed=vt)
+    assert o.dtype == torch.bfloat16
+    ref = N.attention_ref(q, k, v, 1.0 / math.sqrt(d), causal)
+    assert N.rel_l2(o, ref) <= 4e-3 and N.max_abs(o, ref) <= 4e-2, (N.rel_l2(o, ref), N.max_abs(o, ref))
+
+
+def test_bf16_and_fp16_kernels_agree_on_inputs_both_can_hold():
+    # inputs with 3 significant bits are exact in both types: the two kernels then differ only in
+    # how they round the softmax weights and the output
+    g = torch.Generator().manual_seed(77)
+    mk = lambda *shape: (torch.randint(-7, 8, shape, generator=g).float() / 4)
+    q, k, v = mk(2, 256, 128), mk(2, 384, 128), mk(2, 384, 128)
+    o16 = c_attention(q.half().to(DEV), k.half().to(DEV), v.half().to(DEV), causal=True, scale=0.05)
+    ob = c_attention(q.bfloat16().to(DEV), k.bfloat16().to(DEV), v.bfloat16().to(DEV), causal=True, scale=0.05)
+    ref = N.attention_ref(q, k, v, 0.05, True)
+    assert N.rel_l2(o16, ref) <= 1e-3
+    assert N.rel_l2(ob, ref) <= 4e-3
+    assert N.rel_l2(ob.float(), o16.float().cpu()) <= 4e-3

@@ -1,5 +1,5 @@
 // Flash-attention forward for gfx950: O = softmax(scale * Q K^T (+ causal mask)) V per
-// (batch x head) slice, fp16 in/out, fp32 scores and fp32 running max / sum.
+// (batch x head) slice, fp16 or bf16 in/out, fp32 scores and fp32 running max / sum.
 //
 // Counterpart of ke_flash_attention (include/kernels/flash_attention_device.cuh:130-312, mask
 // include/cell/mask.hpp:75-82) and its host launcher (src/kernels/flash_attn.cu:58-152).
@@ -46,19 +46,52 @@ __host__ __device__ constexpr int swz_v(int row, int c) {
 
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 
+// The kernel moves 16-bit elements without looking at them; the element type T (half_t or bf16_t)
+// only selects the MFMA, the float -> T conversion and the dot-product used for the row sums.
+template <typename T>
+struct Vec {
+  using v2 = T __attribute__((ext_vector_type(2)));
+  using v4 = T __attribute__((ext_vector_type(4)));
+  using v8 = T __attribute__((ext_vector_type(8)));
+};
+template <typename T>
+TFK_DEVICE float4_t mfma_t(typename Vec<T>::v8 a, typename Vec<T>::v8 b, float4_t c) {
+  if constexpr (std::is_same_v<T, bf16_t>) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  else return mfma_16x16x32(a, b, c);
+}
+template <typename T>
+TFK_DEVICE float dot2_t(typename Vec<T>::v2 a, typename Vec<T>::v2 b, float c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if constexpr (std::is_same_v<T, bf16_t>) return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false);
+  else return __builtin_amdgcn_fdot2(a, b, c, false);
+#else
+  return c;
+#endif
+}
+// fp16 saturates at its largest finite value (an absurd |Q * scale| must not become inf); bf16
+// has the range of fp32.
+template <typename T>
+TFK_DEVICE T to_elem_saturating(float x) {
+  if constexpr (std::is_same_v<T, bf16_t>) return (T)x;
+  else return (T)__builtin_amdgcn_fmed3f(x, -65504.f, 65504.f);
+}
+
 // `addr` is a 32-bit LDS byte address: integer arithmetic on it (base register + constant)
 // folds into the instruction's offset field, pointer arithmetic through a generic pointer
 // does not.
-TFK_DEVICE half4_t lds_read_tr4(unsigned addr) {
+template <typename V4>
+TFK_DEVICE V4 lds_read_tr4(unsigned addr) {
   fp16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
       (__attribute__((address_space(3))) fp16x4_t*)(size_t)addr);
-  return __builtin_bit_cast(half4_t, v);
+  return __builtin_bit_cast(V4, v);
 }
-TFK_DEVICE half4_t lds_read_b64(unsigned addr) {
-  return *(__attribute__((address_space(3))) const half4_t*)(size_t)addr;
+template <typename V4>
+TFK_DEVICE V4 lds_read_b64(unsigned addr) {
+  return *(__attribute__((address_space(3))) const V4*)(size_t)addr;
 }
-TFK_DEVICE half8_t lds_read_b128(unsigned addr) {
-  return *(__attribute__((address_space(3))) const half8_t*)(size_t)addr;
+template <typename V8>
+TFK_DEVICE V8 lds_read_b128(unsigned addr) {
+  return *(__attribute__((address_space(3))) const V8*)(size_t)addr;
 }
 // Hides how `x` was computed from the optimiser.  Without it the loop-invariant part of
 // (stage base + lane offset + constant) is hoisted as one register per read and the constant
@@ -80,10 +113,13 @@ TFK_DEVICE float quad_sum(float x) {
 // kWavesT wavefronts x 32 queries per workgroup.  8 wavefronts (256 queries) halve the
 // K/V traffic per query and put two wavefronts on every SIMD, so one wavefront's softmax
 // (VALU) overlaps the other's MFMAs; 4 wavefronts serve short query ranges.
-template <int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQB>
+template <typename T, int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQB>
 __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
-    const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V,
-    half_t* __restrict__ O, int Lq, int Lkv, float scale_log2, int q_tiles, int total_items) {
+    const T* __restrict__ Q, const T* __restrict__ K, const T* __restrict__ V,
+    T* __restrict__ O, int Lq, int Lkv, float scale_log2, int q_tiles, int total_items) {
+  using V2 = typename Vec<T>::v2;
+  using V4 = typename Vec<T>::v4;
+  using V8 = typename Vec<T>::v8;
   constexpr int kRowsPerWave = 16 * kQB;  // kQB 16-query blocks per wavefront
   constexpr int kBMq = kWavesT * kRowsPerWave;
   constexpr int kKChunks = D / 8;
@@ -153,16 +189,15 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   // row's reference maximum instead of zero, so the MFMA result IS the exp2 argument - no
   // per-score multiply or subtract is left in the tile loop.
   // Q^T fragments (B operand): lane holds Q'[row][32*kk + 8*lg .. +7]
-  half8_t qf[kKK][kQB];
+  V8 qf[kKK][kQB];
 #pragma unroll
   for (int qb = 0; qb < kQB; ++qb) {
     const int m_ld = min(q_row0 + 16 * qb + lr, Lq - 1);
 #pragma unroll
     for (int kk = 0; kk < kKK; ++kk) {
-      const half8_t raw = *reinterpret_cast<const half8_t*>(Q + (size_t)m_ld * D + kk * 32 + lg * 8);
+      const V8 raw = *reinterpret_cast<const V8*>(Q + (size_t)m_ld * D + kk * 32 + lg * 8);
 #pragma unroll
-      for (int t = 0; t < 8; ++t)   // saturates instead of overflowing to inf for absurd |Q * scale|
-        qf[kk][qb][t] = (half_t)__builtin_amdgcn_fmed3f((float)raw[t] * scale_log2, -65504.f, 65504.f);
+      for (int t = 0; t < 8; ++t) qf[kk][qb][t] = to_elem_saturating<T>((float)raw[t] * scale_log2);
     }
   }
 
@@ -306,25 +341,25 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   // Operand fragments are requested from LDS one step ahead of the MFMAs that use them, into
   // ping-pong registers, so that LDS latency is covered by the previous step's MFMAs (or by
   // the softmax arithmetic) instead of stalling the wavefront in front of every MFMA group.
-  half8_t kf[2][kKB];   // K fragments of reduction step kk (buffer kk & 1)
-  half8_t vf[2][kDB];   // V fragments of reduction step j (buffer j & 1)
+  V8 kf[2][kKB];   // K fragments of reduction step kk (buffer kk & 1)
+  V8 vf[2][kDB];   // V fragments of reduction step j (buffer j & 1)
   auto k_reads = [&](int buf, int it, int kk) __attribute__((always_inline)) {
     const unsigned ka = opaque(smem_base + (it % kStages) * kStageBytes + k_off[kk]);
 #pragma unroll
-    for (int kb = 0; kb < kKB; ++kb) kf[buf][kb] = lds_read_b128(ka + kb * 16 * D * 2);
+    for (int kb = 0; kb < kKB; ++kb) kf[buf][kb] = lds_read_b128<V8>(ka + kb * 16 * D * 2);
   };
   auto v_reads = [&](int buf, int it, int j) __attribute__((always_inline)) {
     const unsigned stage_base = smem_base + (it % kStages) * kStageBytes;
 #pragma unroll
     for (int db = 0; db < kDB; ++db) {
-      half4_t lo, hi;
+      V4 lo, hi;
       if constexpr (!kVT) {
         const unsigned va = opaque(stage_base + v_off[db]) + kKBytes;
-        lo = lds_read_tr4(va + (32 * j) * DV * 2);
-        hi = lds_read_tr4(va + (32 * j + 16) * DV * 2);
+        lo = lds_read_tr4<V4>(va + (32 * j) * DV * 2);
+        hi = lds_read_tr4<V4>(va + (32 * j + 16) * DV * 2);
       } else {
-        lo = lds_read_b64(opaque(stage_base + v_off[2 * j]) + kKBytes + db * 16 * kBN * 2);
-        hi = lds_read_b64(opaque(stage_base + v_off[2 * j + 1]) + kKBytes + db * 16 * kBN * 2);
+        lo = lds_read_b64<V4>(opaque(stage_base + v_off[2 * j]) + kKBytes + db * 16 * kBN * 2);
+        hi = lds_read_b64<V4>(opaque(stage_base + v_off[2 * j + 1]) + kKBytes + db * 16 * kBN * 2);
       }
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -354,11 +389,11 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
       for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
-        for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = mfma_16x16x32(kf[kk & 1][kb], qf[kk][qb], s[kb][qb]);
+        for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = mfma_t<T>(kf[kk & 1][kb], qf[kk][qb], s[kb][qb]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  half8_t pb[kJ][kQB];  // fp16 weights, B operand of the second product
+  V8 pb[kJ][kQB];  // 16-bit weights, B operand of the second product
   // ---- mask, online softmax, fp16 weights.  Requests the V fragments of step j = 0. -------
   auto softmax_tile = [&](int it, auto mask_c) __attribute__((always_inline)) {
     constexpr bool kMask = decltype(mask_c)::value;
@@ -423,21 +458,21 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 
     // The row sum is taken over the fp16-rounded weights, the values that actually multiply
     // V (v_dot2_f32_f16 against (1, 1): two weights per instruction, fp32 accumulate).
-    const half2_t ones = {(half_t)1.f, (half_t)1.f};
+    const V2 ones = {(T)1.f, (T)1.f};
 #pragma unroll
     for (int j = 0; j < kJ; ++j)
 #pragma unroll
       for (int qb = 0; qb < kQB; ++qb) {
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          pb[j][qb][t] = (half_t)s[2 * j][qb][t];
-          pb[j][qb][4 + t] = (half_t)s[2 * j + 1][qb][t];
+          pb[j][qb][t] = (T)s[2 * j][qb][t];
+          pb[j][qb][4 + t] = (T)s[2 * j + 1][qb][t];
         }
         float ps = l_run[qb];
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 0, 1), ones, ps, false);
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 2, 3), ones, ps, false);
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 4, 5), ones, ps, false);
-        ps = __builtin_amdgcn_fdot2(__builtin_shufflevector(pb[j][qb], pb[j][qb], 6, 7), ones, ps, false);
+        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 0, 1), ones, ps);
+        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 2, 3), ones, ps);
+        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 4, 5), ones, ps);
+        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 6, 7), ones, ps);
         l_run[qb] = ps;
       }
     __builtin_amdgcn_sched_barrier(0);
@@ -452,7 +487,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
       for (int db = 0; db < kDB; ++db)
 #pragma unroll
-        for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = mfma_16x16x32(vf[j & 1][db], pb[j][qb], o_acc[db][qb]);
+        for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = mfma_t<T>(vf[j & 1][db], pb[j][qb], o_acc[db][qb]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -532,15 +567,14 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     for (int qb = 0; qb < kQB; ++qb) {
       const float inv = 1.f / quad_sum(l_run[qb]);   // of this lane's own row lr
       const int m_row = q_row0 + 16 * qb + st_row;   // the row this lane stores
-      half_t* o_lane = O + (size_t)m_row * DV + 8 * st_seg;
+      T* o_lane = O + (size_t)m_row * DV + 8 * st_seg;
 #pragma unroll
       for (int db = 0; db < kDB; db += 2) {
-        typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
         unsigned x[2], y[2];
 #pragma unroll
         for (int d = 0; d < 2; ++d) {
-          const h2_t hx = {(half_t)(o_acc[db][qb][2 * d] * inv), (half_t)(o_acc[db][qb][2 * d + 1] * inv)};
-          const h2_t hy = {(half_t)(o_acc[db + 1][qb][2 * d] * inv), (half_t)(o_acc[db + 1][qb][2 * d + 1] * inv)};
+          const V2 hx = {(T)(o_acc[db][qb][2 * d] * inv), (T)(o_acc[db][qb][2 * d + 1] * inv)};
+          const V2 hy = {(T)(o_acc[db + 1][qb][2 * d] * inv), (T)(o_acc[db + 1][qb][2 * d + 1] * inv)};
           x[d] = __builtin_bit_cast(unsigned, hx);
           y[d] = __builtin_bit_cast(unsigned, hy);
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -564,10 +598,10 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   }  // pass
 }
 
-template <int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQB>
+template <typename T, int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQB>
 int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
              float scale_log2, hipStream_t st) {
-  auto kern = flash_attention_fwd_kernel<D, DV, kVT, kCausal, kWavesT, kQB>;
+  auto kern = flash_attention_fwd_kernel<T, D, DV, kVT, kCausal, kWavesT, kQB>;
   constexpr int lds = kStages * (kBN * D * 2 + kBN * DV * 2);
   static_assert(lds <= kMaxLdsBytes, "tiles do not fit in LDS");
   TFK_LDS_OPT_IN(kern, lds);
@@ -577,29 +611,29 @@ int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, in
   const int total_items = (kCausal && q_tiles % 2 == 0) ? (q_tiles / 2) * batch : q_tiles * batch;
   const dim3 grid(8 * ((total_items + 7) / 8));
   hipLaunchKernelGGL(kern, grid, dim3(kWavesT * 64), lds, st,
-                     static_cast<const half_t*>(Q), static_cast<const half_t*>(K),
-                     static_cast<const half_t*>(V), static_cast<half_t*>(O), Lq, Lkv, scale_log2,
+                     static_cast<const T*>(Q), static_cast<const T*>(K),
+                     static_cast<const T*>(V), static_cast<T*>(O), Lq, Lkv, scale_log2,
                      q_tiles, total_items);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
 }
 
-template <int D, int DV, bool kVT, bool kCausal>
+template <typename T, int D, int DV, bool kVT, bool kCausal>
 int launch(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
            float scale_log2, hipStream_t st) {
-  if (Lq > 128) return launch_w<D, DV, kVT, kCausal, 8, 2>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
-  return launch_w<D, DV, kVT, kCausal, 4, 2>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+  if (Lq > 128) return launch_w<T, D, DV, kVT, kCausal, 8, 2>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+  return launch_w<T, D, DV, kVT, kCausal, 4, 2>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
 }
 
-template <int D, int DV>
+template <typename T, int D, int DV>
 int pick(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
          float scale_log2, bool vt, bool causal, hipStream_t st) {
   if (vt) {
-    if (causal) return launch<D, DV, true, true>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
-    return launch<D, DV, true, false>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+    if (causal) return launch<T, D, DV, true, true>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+    return launch<T, D, DV, true, false>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
   }
-  if (causal) return launch<D, DV, false, true>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
-  return launch<D, DV, false, false>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+  if (causal) return launch<T, D, DV, false, true>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
+  return launch<T, D, DV, false, false>(Q, K, V, O, batch, Lq, Lkv, scale_log2, st);
 }
 
 }  // namespace
@@ -661,10 +695,10 @@ extern "C" int tf_flash_attention_fwd_f16(const void* Q, const void* K, const vo
               "tf_flash_attention_fwd_f16: transposed V needs Lkv %% 8 == 0");
   const float scale_log2 = (float)(softmax_scale * 1.4426950408889634);
   if (D == 128)
-    return pick<128, 128>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
-                          v_is_transposed != 0, causal != 0, st);
-  return pick<64, 64>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
-                      v_is_transposed != 0, causal != 0, st);
+    return pick<half_t, 128, 128>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
+                                  v_is_transposed != 0, causal != 0, st);
+  return pick<half_t, 64, 64>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
+                              v_is_transposed != 0, causal != 0, st);
 }
 
 extern "C" int tf_flash_attention_fwd(const void* Q, const void* K, const void* V, void* O, int dtype, int64_t batch,
@@ -680,7 +714,16 @@ extern "C" int tf_flash_attention_fwd(const void* Q, const void* K, const void* 
   if (int rc = check_attention_args("tf_flash_attention_fwd", Q, K, V, O, batch, Lq, Lkv, D, Dv, tile_length_q,
                                     tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale))
     return rc;
-  return attention_fallback("tf_flash_attention_fwd", Q, K, V, O, dtype, batch, Lq, Lkv, D, Dv, v_is_transposed,
-                            tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale, causal,
-                            static_cast<hipStream_t>(stream));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool tuned = ((D == 128 && Dv == 128) || (D == 64 && Dv == 64)) && (!v_is_transposed || Lkv % 8 == 0);
+  if (!tuned)
+    return attention_fallback("tf_flash_attention_fwd", Q, K, V, O, dtype, batch, Lq, Lkv, D, Dv, v_is_transposed,
+                              tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale, causal, st);
+  // the tuned kernels with the bf16 MFMA, bf16 weights and bf16 output
+  const float scale_log2 = (float)(softmax_scale * 1.4426950408889634);
+  if (D == 128)
+    return pick<bf16_t, 128, 128>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
+                                  v_is_transposed != 0, causal != 0, st);
+  return pick<bf16_t, 64, 64>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
+                              v_is_transposed != 0, causal != 0, st);
 }
