@@ -79,3 +79,18 @@ def test_header_kernel_gemm_table_is_correct():
     buf = io.StringIO()
     assert mod.run(out=buf), buf.getvalue()
     assert "MISMATCH" not in buf.getvalue()
+
+
+def test_attention_head_dim_table_is_correct_on_a_small_problem():
+    import importlib.util
+
+    import torch
+
+    spec = importlib.util.spec_from_file_location("attn_bench", os.path.join(ROOT, "benchmarks", "attention", "bench.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    buf = io.StringIO()
+    cases = [(128, torch.float16, True, "tuned"), (64, torch.bfloat16, False, "tuned"),
+             (96, torch.float16, True, "header kernel"), (32, torch.bfloat16, False, "header kernel")]
+    assert mod.run(cases=cases, bh=2, s=512, out=buf), buf.getvalue()
+    assert "MISMATCH" not in buf.getvalue()

@@ -9,6 +9,13 @@
 // entirely above the diagonal.  exp(S - max) is rounded to fp16 and re-laid-out through an LDS
 // tile for the second MFMA.  (The library's tuned entry point tf_flash_attention_fwd_f16
 // computes the scores transposed instead and needs no re-layout.)
+//
+// When one k-chunk covers the whole head dimension (kTK == kK) the Q tile is fetched once and
+// stays in registers (the reference reloads it per key tile,
+// include/kernels/flash_attention_device.cuh:231-262).  K / V tiles keep one LDS buffer each:
+// double-buffering them was measured and loses more to the lower occupancy (two instead of three
+// workgroups per CU at a head dimension of 96) than the overlap gains, because co-resident
+// workgroups already cover each other's loads.
 #pragma once
 
 #include "cell/mod.hpp"
@@ -98,6 +105,8 @@ struct FlashAttentionTraits {
   using ApplyMask = cell::ApplyMask<RegAcc, WarpLayout, BaseShape, MaskMode::kCausal>;
   using ApplyScoreScale = compute::BroadcastScalarMul<RegAcc>;
 
+  // the whole head dimension in one chunk: Q is fetched once (see above)
+  static constexpr bool kWholeK = kTK == kK;
   static constexpr int kSharedBytes =
       (SharedQ::kNumel + SharedK::kNumel + SharedV::kNumel + SharedP::kNumel) * (int)sizeof(InType);
 };
@@ -143,18 +152,8 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
   // causal: key tiles that start after the last row of this workgroup contribute nothing
   const int n_tiles = T::kIsCausal ? min((int)T::GIteratorV::sc0, (row_base + kTM + kTN - 1) / kTN)
                                    : (int)T::GIteratorV::sc0;
-  for (int n = 0; n < n_tiles; ++n) {
-    load_sv(gVs(n), sV);
-    for (int k = 0; k < T::GIteratorQ::sc1; ++k) {
-      load_sq(gQs(k), sQ);
-      load_sk(gKs(k, n), sK);
-      __copy_async();
-      __syncthreads();
-      load_rq(sQ, rQ);
-      load_rk(sK, rK);
-      compute::gemm(rQ, rK, s);
-      __syncthreads();
-    }
+  // scale, mask, online softmax of the score tile `s` of key tile n; leaves the fp16 weights in sP
+  auto softmax_tile = [&](int n) {
     typename T::ApplyScoreScale scale;
     scale(s, AccType(T::kSoftmaxScale), s);
     if constexpr (T::kIsCausal) {
@@ -191,14 +190,50 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
     to_half(s, p_half);
     typename T::StorerP store_p;
     store_p(p_half, sP);
-    __copy_async();
-    __syncthreads();
-    typename T::LoaderP load_p;
-    load_p(sP, rP);
-    load_rv(sV, rV);
-    compute::gemm(rP, rV, o);
-    s.clear();
-    __syncthreads();
+  };
+
+  if constexpr (T::kWholeK) {
+    load_sq(gQs(0), sQ);
+    for (int n = 0; n < n_tiles; ++n) {
+      load_sk(gKs(0, n), sK);
+      load_sv(gVs(n), sV);
+      __copy_async();
+      __syncthreads();
+      if (n == 0) load_rq(sQ, rQ);   // stays in registers for every key tile
+      load_rk(sK, rK);
+      compute::gemm(rQ, rK, s);
+      softmax_tile(n);
+      __syncthreads();   // the weights are in LDS
+      typename T::LoaderP load_p;
+      load_p(sP, rP);
+      load_rv(sV, rV);
+      compute::gemm(rP, rV, o);
+      s.clear();
+      __syncthreads();   // nobody still reads this tile or its weights
+    }
+  } else {
+    for (int n = 0; n < n_tiles; ++n) {
+      load_sv(gVs(n), sV);
+      for (int k = 0; k < T::GIteratorQ::sc1; ++k) {
+        load_sq(gQs(k), sQ);
+        load_sk(gKs(k, n), sK);
+        __copy_async();
+        __syncthreads();
+        load_rq(sQ, rQ);
+        load_rk(sK, rK);
+        compute::gemm(rQ, rK, s);
+        __syncthreads();
+      }
+      softmax_tile(n);
+      __copy_async();
+      __syncthreads();
+      typename T::LoaderP load_p;
+      load_p(sP, rP);
+      load_rv(sV, rV);
+      compute::gemm(rP, rV, o);
+      s.clear();
+      __syncthreads();
+    }
   }
   typename T::BroadcastDiv normalise;
   normalise(run_sum, o);
