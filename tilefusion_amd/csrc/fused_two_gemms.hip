@@ -163,31 +163,44 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
   C += batch * (size_t)P * N;
   D += batch * (size_t)M * P;
 
-  const int a_row = min(m0 + wave * 16 + lr, M - 1);  // clamped: rows past M are never stored
-  const half_t* a_ptr = A + (size_t)a_row * K + 8 * lg;
+  // Every global access is a scalar base (tile origin, 64-bit, computed on the scalar unit) plus
+  // a 32-bit byte offset per lane that stays inside the tile: the address arithmetic in front of
+  // the first request is on this kernel's critical path (per-lane 64-bit pointers for the 4 + 16
+  // requests of a wavefront cost ~1 us of the ~3.5 us the kernel ran).
+  const int a_row = min(wave * 16 + lr, M - 1 - m0);  // clamped: rows past M are never stored
+  const char* a_base = reinterpret_cast<const char*>(A + (size_t)m0 * K);
+  const unsigned a_off = ((unsigned)a_row * (unsigned)K + 8u * lg) * 2u;
   const unsigned sB_addr = lds_address(sB), sC_addr = lds_address(sC);
+  auto dma = [](unsigned off, const char* base, unsigned lds_addr) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(off), "s"(base), "s"(lds_addr)
+                 : "memory");
+  };
 
   // 1 KiB request i of the B tile covers rows 64 / kBCh * i ..; lane l fills physical chunk
   // l % kBCh of its row with the logical chunk the key maps there.  The same for C with the
   // plain key.  Requests beyond the tile (a C tile smaller than 1 KiB) re-fetch row 0.
   auto request_b = [&](int n0, int k0) __attribute__((always_inline)) {
+    const char* b_base = reinterpret_cast<const char*>(B + (size_t)n0 * K + k0);
 #pragma unroll
     for (int q = 0; q < kBPerWave; ++q) {
       const int i = wave + kWaves * q;
       if (kBInstr % kWaves != 0 && i >= kBInstr) break;
       const int row = i * (64 / kBCh) + lane / kBCh;
       const int c = (lane % kBCh) ^ b_key<kBCh>(row);
-      lds_dma_16B(B + (size_t)(n0 + row) * K + k0 + c * 8, sB_addr + i * 1024);
+      dma(((unsigned)row * (unsigned)K + (unsigned)c * 8u) * 2u, b_base, sB_addr + i * 1024);
     }
   };
   auto request_c = [&](int n0) __attribute__((always_inline)) {
+    const char* c_base = reinterpret_cast<const char*>(C + (size_t)p0 * N + n0);
 #pragma unroll
     for (int q = 0; q < kCPerWave; ++q) {
       const int i = wave + kWaves * q;
       if (kCInstr % kWaves != 0 && i >= kCInstr) break;
       const int row = min(i * (64 / kCCh) + lane / kCCh, TP - 1);
       const int c = swz<kCCh>(row, lane % kCCh);
-      lds_dma_16B(C + (size_t)(p0 + row) * N + n0 + c * 8, sC_addr + i * 1024);
+      dma(((unsigned)row * (unsigned)N + (unsigned)c * 8u) * 2u, c_base, sC_addr + i * 1024);
     }
   };
   // requests of this wavefront that are still allowed in flight when B (and A) must be there
@@ -225,9 +238,17 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
       // All three kinds of request are issued from assembly, so that the compiler places no
       // vector-memory waits of its own (it would drain everything, the C tile included, in
       // front of the first LDS read or the first use of an A fragment).
+      {
+        const char* a_chunk = a_base + (size_t)k0 * 2;
 #pragma unroll
-      for (int ks = 0; ks < kKSteps; ++ks)
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(af[ks]) : "v"(a_ptr + k0 + ks * 32) : "memory");
+        for (int ks = 0; ks < kKSteps; ++ks)
+          asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3"
+                       : "=v"(af[ks])
+                       : "v"(a_off), "s"(a_chunk), "n"(ks * 64)
+                       : "memory");
+      }
+      // the A requests are on their way before the arithmetic of the B and C requests starts
+      __builtin_amdgcn_sched_barrier(0);
       request_b(n0, k0);
       if (first_chunk) request_c(n0);
       // A and B have landed once at most this wavefront's C requests are outstanding (loads
