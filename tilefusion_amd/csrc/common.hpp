@@ -80,6 +80,10 @@ TFK_DEVICE void barrier_keep_vmem() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+// Bare workgroup barrier: nothing of this wavefront is drained (LDS reads and vector-memory loads
+// stay in flight; the caller knows that nothing another wavefront does behind it depends on them).
+TFK_DEVICE void barrier_only() { asm volatile("s_barrier" ::: "memory"); }
+
 // Workgroup barrier that only drains this wavefront's LDS traffic (reads and writes), leaving
 // global loads into registers in flight.
 TFK_DEVICE void barrier_lds_only() {

@@ -27,7 +27,9 @@ namespace tfk {
 namespace {
 
 constexpr int kBN = 64;   // keys per tile
-constexpr int kStages = 4;
+// LDS ring depth: the 8-wavefront kernel keeps two tiles live (its two wavefront sets are half a
+// tile apart) and three in flight; the 4-wavefront kernel one live and three in flight.
+__host__ __device__ constexpr int ring_stages(int waves) { return waves == 8 ? 5 : 4; }
 
 // K tile [kBN][D] (and a transposed V tile [DV][kBN]): 16 consecutive rows reading one logical
 // 16-byte chunk hit 16 different bank groups.
@@ -47,7 +49,7 @@ __host__ __device__ constexpr int swz_v(int row, int c) {
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 
 // The kernel moves 16-bit elements without looking at them; the element type T (half_t or bf16_t)
-// only selects the MFMA, the float -> T conversion and the dot-product used for the row sums.
+// only selects the MFMA and the float -> T conversion.
 template <typename T>
 struct Vec {
   using v2 = T __attribute__((ext_vector_type(2)));
@@ -58,15 +60,6 @@ template <typename T>
 TFK_DEVICE float4_t mfma_t(typename Vec<T>::v8 a, typename Vec<T>::v8 b, float4_t c) {
   if constexpr (std::is_same_v<T, bf16_t>) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   else return mfma_16x16x32(a, b, c);
-}
-template <typename T>
-TFK_DEVICE float dot2_t(typename Vec<T>::v2 a, typename Vec<T>::v2 b, float c) {
-#if defined(__HIP_DEVICE_COMPILE__)
-  if constexpr (std::is_same_v<T, bf16_t>) return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false);
-  else return __builtin_amdgcn_fdot2(a, b, c, false);
-#else
-  return c;
-#endif
 }
 // fp16 saturates at its largest finite value (an absurd |Q * scale| must not become inf); bf16
 // has the range of fp32.
@@ -100,14 +93,10 @@ TFK_DEVICE unsigned opaque(unsigned x) {
   asm volatile("" : "+v"(x));
   return x;
 }
-// Reductions over the 4 lanes l, l^16, l^32, l^48 that share a query (rare path / epilogue).
+// Reduction over the 4 lanes l, l^16, l^32, l^48 that share a query (rare path).
 TFK_DEVICE float quad_max(float x) {
   x = fmaxf(x, __shfl_xor(x, 16));
   return fmaxf(x, __shfl_xor(x, 32));
-}
-TFK_DEVICE float quad_sum(float x) {
-  x += __shfl_xor(x, 16);
-  return x + __shfl_xor(x, 32);
 }
 
 // kWavesT wavefronts x 32 queries per workgroup.  8 wavefronts (256 queries) halve the
@@ -120,6 +109,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   using V2 = typename Vec<T>::v2;
   using V4 = typename Vec<T>::v4;
   using V8 = typename Vec<T>::v8;
+  constexpr int kStages = ring_stages(kWavesT);
   constexpr int kRowsPerWave = 16 * kQB;  // kQB 16-query blocks per wavefront
   constexpr int kBMq = kWavesT * kRowsPerWave;
   constexpr int kKChunks = D / 8;
@@ -266,6 +256,21 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       }
     }
   };
+  // The same request for a tile known to lie wholly inside the key range: no clamping, no
+  // branch.  The tile loop uses this form wherever it can, because the bookkeeping of the
+  // general form (~30 scalar instructions and two branches per request) is issued between
+  // MFMAs of a wavefront that has the matrix pipe to itself at that moment: it cost ~100
+  // cycles per request with the pipe idle.
+  auto issue_request_lean = [&](int tile, int r) __attribute__((always_inline)) {
+    const unsigned dst = smem_base + (tile % kStages) * kStageBytes + req_lds[r];
+    const char* base = r < kKPerWave ? reinterpret_cast<const char*>(K) + (size_t)tile * (kBN * D * 2)
+                       : kVT         ? reinterpret_cast<const char*>(V) + (size_t)tile * (kBN * 2)
+                                     : reinterpret_cast<const char*>(V) + (size_t)tile * (kBN * DV * 2);
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(req_off[r]), "s"(base), "s"(dst)
+                 : "memory");
+  };
   auto issue_tile_loads = [&](int tile) __attribute__((always_inline)) {
 #pragma unroll
     for (int r = 0; r < kLoadsPerTile; ++r) issue_request(tile, r);
@@ -311,33 +316,23 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
     for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = float4_t{0.f, 0.f, 0.f, 0.f};
   // neg_m: minus the reference maximum of a row's scaled scores (the accumulator start value);
-  // l_run: this lane's share of the running sum of weights.
-  float neg_m[kQB], l_run[kQB];
+  // l_acc: the running sum of a row's weights, kept as one more accumulator block of the second
+  // product (a block of V^T whose 16 rows are all ones): the matrix pipe adds up the 16-bit
+  // weights that actually multiply V.  Every register of l_acc[qb] holds the sum of row lr.
+  // (A v_dot2 per pair of weights, the obvious VALU form, takes ~20 cycles per instruction while
+  // another wavefront of the SIMD streams MFMAs - against 8 for an ordinary VALU instruction.)
+  float neg_m[kQB];
+  float4_t l_acc[kQB];
 #pragma unroll
   for (int qb = 0; qb < kQB; ++qb) {
     neg_m[qb] = 0.f;  // reference 0 until the first tile raises it
-    l_run[qb] = 0.f;
+    l_acc[qb] = float4_t{0.f, 0.f, 0.f, 0.f};
   }
-
-  // Ring of kStages tiles.  Iteration `it` starts with the ring barrier: wait until tile it+1
-  // has landed (only the loads of younger tiles stay in flight) and meet the other wavefronts;
-  // after it the stage of tile it-1 is free and tile it+kStages-1 is requested into it.  Tile
-  // it+1 is needed that early because the wavefronts of a workgroup run in two phases (below).
-  // The requests are NOT issued in one burst behind the barrier: eight wavefronts handing 32
-  // KiB of requests to the CU's one address unit at the same moment all stall in the issue
-  // queue with the matrix pipe idle (measured: ~500 of 4100 cycles per tile).  They ride along
-  // with the MFMAs of the next QK product instead, one request per reduction step.
+  V8 ones_frag;
 #pragma unroll
-  for (int t = 0; t < kStages - 1; ++t) issue_tile_loads(t);
-  barrier_keep_vmem<(kStages - 2) * kLoadsPerTile>();  // tile 0 has landed
-  auto ring_barrier = [&]() __attribute__((always_inline)) {
-    barrier_keep_vmem<(kStages - 3) * kLoadsPerTile>();
-  };
-  auto ring_step = [&](int it) __attribute__((always_inline)) {  // burst form, off the hot path
-    ring_barrier();
-    issue_tile_loads(it + kStages - 1);
-  };
-  float4_t s[kKB][kQB];  // scores of the tile in flight (carried across iterations by late wavefronts)
+  for (int t = 0; t < 8; ++t) ones_frag[t] = (T)1.f;
+
+  float4_t s[kKB][kQB];  // scores of the tile in flight
   // Operand fragments are requested from LDS one step ahead of the MFMAs that use them, into
   // ping-pong registers, so that LDS latency is covered by the previous step's MFMAs (or by
   // the softmax arithmetic) instead of stalling the wavefront in front of every MFMA group.
@@ -372,25 +367,35 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   //      against row lr of query block qb, minus that row's reference maximum.  Expects the
   //      fragments of step kk = 0 to be on their way into kf[0]. ---------------------------
   //      req_tile >= 0: that tile's requests are issued between the reduction steps.
-  auto qk_tile = [&](int it, int req_tile) __attribute__((always_inline)) {
+  //      lean_c: the requested tile is a whole tile inside the key range (lean request form).
+  //      The fragment reads of the next reduction step and the requests sit BETWEEN the MFMAs
+  //      (one piece behind each pair): a wavefront issues in order, so anything clustered
+  //      between two reduction steps runs with the matrix pipe drained.
+  auto qk_tile = [&](int it, int req_tile, auto lean_c) __attribute__((always_inline)) {
+    constexpr bool kLean = decltype(lean_c)::value;
 #pragma unroll
     for (int kb = 0; kb < kKB; ++kb)
 #pragma unroll
       for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = float4_t{neg_m[qb], neg_m[qb], neg_m[qb], neg_m[qb]};
 #pragma unroll
     for (int kk = 0; kk < kKK; ++kk) {
-      if (kk + 1 < kKK) k_reads((kk + 1) & 1, it, kk + 1);
-      if (req_tile >= 0) {
-#pragma unroll
-        for (int r = 0; r < kLoadsPerTile; ++r)
-          if ((r * kKK) / kLoadsPerTile == kk) issue_request(req_tile, r);
-      }
+      const unsigned ka = kk + 1 < kKK ? opaque(smem_base + (it % kStages) * kStageBytes + k_off[kk + 1]) : 0u;
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int kb = 0; kb < kKB; ++kb)
+      for (int kb = 0; kb < kKB; ++kb) {
 #pragma unroll
         for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = mfma_t<T>(kf[kk & 1][kb], qf[kk][qb], s[kb][qb]);
-      __builtin_amdgcn_sched_barrier(0);
+        if (kk + 1 < kKK) kf[(kk + 1) & 1][kb] = lds_read_b128<V8>(ka + kb * 16 * D * 2);
+        if (req_tile >= 0) {
+#pragma unroll
+          for (int r = 0; r < kLoadsPerTile; ++r)
+            if ((r * kKK * kKB) / kLoadsPerTile == kk * kKB + kb) {
+              if constexpr (kLean) issue_request_lean(req_tile, r);
+              else issue_request(req_tile, r);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
   V8 pb[kJ][kQB];  // 16-bit weights, B operand of the second product
@@ -441,7 +446,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
         const float qmax = quad_max(mx[qb]);
         const float shift = first ? qmax : fmaxf(0.f, qmax);  // afterwards the reference only rises
         const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-shift);
-        l_run[qb] *= alpha;
+        l_acc[qb] *= alpha;
 #pragma unroll
         for (int db = 0; db < kDB; ++db) o_acc[db][qb] *= alpha;
 #pragma unroll
@@ -456,9 +461,6 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) s[kb][qb][r] = __builtin_amdgcn_exp2f(s[kb][qb][r]);
 
-    // The row sum is taken over the fp16-rounded weights, the values that actually multiply
-    // V (v_dot2_f32_f16 against (1, 1): two weights per instruction, fp32 accumulate).
-    const V2 ones = {(T)1.f, (T)1.f};
 #pragma unroll
     for (int j = 0; j < kJ; ++j)
 #pragma unroll
@@ -468,12 +470,6 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
           pb[j][qb][t] = (T)s[2 * j][qb][t];
           pb[j][qb][4 + t] = (T)s[2 * j + 1][qb][t];
         }
-        float ps = l_run[qb];
-        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 0, 1), ones, ps);
-        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 2, 3), ones, ps);
-        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 4, 5), ones, ps);
-        ps = dot2_t<T>(__builtin_shufflevector(pb[j][qb], pb[j][qb], 6, 7), ones, ps);
-        l_run[qb] = ps;
       }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -488,6 +484,8 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       for (int db = 0; db < kDB; ++db)
 #pragma unroll
         for (int qb = 0; qb < kQB; ++qb) o_acc[db][qb] = mfma_t<T>(vf[j & 1][db], pb[j][qb], o_acc[db][qb]);
+#pragma unroll
+      for (int qb = 0; qb < kQB; ++qb) l_acc[qb] = mfma_t<T>(ones_frag, pb[j][qb], l_acc[qb]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -501,53 +499,88 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     n_plain = max(0, min(n_plain, (q_row0 + 1) / kBN));
     n_compute = min(num_tiles, (q_row0 + kRowsPerWave - 1) / kBN + 1);
   }
-  // Two wavefronts share a SIMD (w and w + 4).  If both ran QK -> softmax -> PV in lockstep
-  // (the per-tile barrier aligns them), they would fight for the MFMA pipe in two phases and
-  // leave it idle while both do their softmax.  So the second wavefront of each SIMD runs one
-  // phase late - softmax(it), PV(it), QK(it+1) between the same barriers - and its softmax
-  // overlaps the first one's QK MFMAs, the first one's softmax its PV MFMAs.
-  const bool late = kWavesT == 8 && wave >= 4;
-  int it = 0;
-  k_reads(0, 0, 0);
-  if (!late) {
-    for (; it < n_plain; ++it) {
-      ring_barrier();
-      qk_tile(it, it + kStages - 1);
-      softmax_tile(it, std::false_type{});
-      pv_tile(it, it + 1);
-    }
-    for (; it < n_compute; ++it) {
-      ring_barrier();
-      qk_tile(it, it + kStages - 1);
-      softmax_tile(it, std::true_type{});
-      pv_tile(it, it + 1);
-    }
-  } else {
-    // The issue arbiter prefers the older wavefront: when this wavefront's QK product meets
-    // the first one's PV product on the MFMA pipe it would lose every slot, reach the barrier
-    // ~700 cycles after the first one (measured with s_memtime) and finish its product alone
-    // with the other wavefront idle.  Raised priority for that one product evens them out.
-    auto late_qk = [&](int it_) __attribute__((always_inline)) {
-      __builtin_amdgcn_s_setprio(2);
-      if (it_ + 1 < n_compute) qk_tile(it_ + 1, it_ + kStages - 1);
-      else issue_tile_loads(it_ + kStages - 1);
-      __builtin_amdgcn_s_setprio(0);
+  const int n_fast = min(num_tiles, Lkv / kBN);  // whole tiles of this pass (lean request form)
+  if constexpr (kWavesT == 8) {
+    // Two wavefronts share a SIMD (w and w + 4) and a SIMD has one matrix pipe and one VALU, so
+    // the two SETS of wavefronts (0-3, 4-7) run the same loop half a tile apart, in time slots
+    // fenced by two workgroup barriers per tile:
+    //     slot 2t   : set 0: PV(t-1), QK(t)  [MFMA]      set 1: softmax(t-1)     [VALU]
+    //     slot 2t+1 : set 0: softmax(t)      [VALU]      set 1: PV(t-1), QK(t)   [MFMA]
+    // While one wavefront of a SIMD streams its 64 MFMAs the other one does its exp2 / convert
+    // work, and neither pipe waits for the other: measured per tile, a wavefront's MFMA block
+    // takes ~1100-1200 cycles and its softmax ~1000 while the partner's MFMAs run (VALU
+    // instructions issue at half rate then), against ~3500 for an arrangement that lets the
+    // phases of the two wavefronts drift (QK, softmax and PV of both then run one after another).
+    // Without the second barrier the sets do drift: the hardware issues from the older wavefront
+    // first and whichever set gets ahead keeps the matrix pipe.
+    // Ring of 5 tiles: tile t is read from slot 2t (QK by set 0) to slot 2t+3 (PV by set 1), so
+    // two tiles are live and three are in flight.  QK(t) carries the requests of tile t+3, which
+    // go into the stage of tile t-2 (last read in slot 2t-1).  The barrier behind an MFMA block
+    // (after QK(t+1) has requested tile t+4) waits until only tiles t+3, t+4 are in flight: tile
+    // t+2 has then landed, one slot before the first wavefront reads it.
+#pragma unroll
+    for (int t = 0; t < 3; ++t) issue_tile_loads(t);
+    barrier_keep_vmem<2 * kLoadsPerTile>();  // tile 0 has landed
+    const bool second_set = wave >= 4;
+    if (second_set) barrier_only();  // slot 0: set 0 alone
+    k_reads(0, 0, 0);
+    if (n_compute > 0) qk_tile(0, 3, std::false_type{});
+    else issue_tile_loads(3);
+    auto tile_step = [&](int t, auto mask_c, auto lean_c) __attribute__((always_inline)) {
+      barrier_keep_vmem<2 * kLoadsPerTile>();  // tile t+1 has landed (own loads; then everyone's)
+      softmax_tile(t, mask_c);
+      barrier_only();  // the V fragments requested by softmax_tile stay in flight across it
+      pv_tile(t, t + 1);
+      if (t + 1 < n_compute) qk_tile(t + 1, t + 4, lean_c);
+      else issue_tile_loads(t + 4);
     };
-    qk_tile(0, -1);
-    for (; it < n_plain; ++it) {
+    // [0, n_lean): unmasked tile, a QK product follows and its requests (tile t+4) are whole tiles
+    const int n_lean = min(min(n_plain, n_compute - 1), n_fast - 4);
+    int t = 0;
+    for (; t < n_lean; ++t) tile_step(t, std::false_type{}, std::true_type{});
+    for (; t < n_plain; ++t) tile_step(t, std::false_type{}, std::false_type{});
+    for (; t < n_compute; ++t) tile_step(t, std::true_type{}, std::false_type{});
+    for (; t < num_tiles; ++t) {  // above the diagonal: keep the ring and the barriers going
+      barrier_keep_vmem<2 * kLoadsPerTile>();
+      barrier_only();
+      issue_tile_loads(t + 4);
+    }
+    if (!second_set) barrier_only();  // the slot in which set 1 finishes its last tile
+  } else {
+    // One wavefront per SIMD.  Ring of 4 tiles: iteration `it` starts with the ring barrier (tile
+    // it has landed, the stage of tile it-1 is free) and QK(it) carries the requests of tile it+3.
+#pragma unroll
+    for (int t = 0; t < kStages - 1; ++t) issue_tile_loads(t);
+    barrier_keep_vmem<(kStages - 2) * kLoadsPerTile>();  // tile 0 has landed
+    auto ring_barrier = [&]() __attribute__((always_inline)) {
+      barrier_keep_vmem<(kStages - 3) * kLoadsPerTile>();
+    };
+    const int n_lean = min(n_plain, n_fast - (kStages - 1));
+    int it = 0;
+    k_reads(0, 0, 0);
+    for (; it < n_lean; ++it) {
       ring_barrier();
+      qk_tile(it, it + kStages - 1, std::true_type{});
       softmax_tile(it, std::false_type{});
       pv_tile(it, it + 1);
-      late_qk(it);
+    }
+    for (; it < n_plain; ++it) {
+      ring_barrier();
+      qk_tile(it, it + kStages - 1, std::false_type{});
+      softmax_tile(it, std::false_type{});
+      pv_tile(it, it + 1);
     }
     for (; it < n_compute; ++it) {
       ring_barrier();
+      qk_tile(it, it + kStages - 1, std::false_type{});
       softmax_tile(it, std::true_type{});
       pv_tile(it, it + 1);
-      late_qk(it);
+    }
+    for (; it < num_tiles; ++it) {
+      ring_barrier();
+      issue_tile_loads(it + kStages - 1);
     }
   }
-  for (; it < num_tiles; ++it) ring_step(it);
   wait_vmem_all();  // the clamped tail loads must not outlive the workgroup's LDS
 
   // ---- epilogue: O[m][16*db + 4*lg + r] = O^T / l ------------------------------------------
@@ -565,7 +598,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     const int src_lane = st_row + 16 * (((st_seg & 1) << 1) | (st_seg >> 1));
 #pragma unroll
     for (int qb = 0; qb < kQB; ++qb) {
-      const float inv = 1.f / quad_sum(l_run[qb]);   // of this lane's own row lr
+      const float inv = 1.f / l_acc[qb][0];   // of this lane's own row lr
       const int m_row = q_row0 + 16 * qb + st_row;   // the row this lane stores
       T* o_lane = O + (size_t)m_row * DV + 8 * st_seg;
 #pragma unroll
@@ -602,7 +635,7 @@ template <typename T, int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQ
 int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
              float scale_log2, hipStream_t st) {
   auto kern = flash_attention_fwd_kernel<T, D, DV, kVT, kCausal, kWavesT, kQB>;
-  constexpr int lds = kStages * (kBN * D * 2 + kBN * DV * 2);
+  constexpr int lds = ring_stages(kWavesT) * (kBN * D * 2 + kBN * DV * 2);
   static_assert(lds <= kMaxLdsBytes, "tiles do not fit in LDS");
   TFK_LDS_OPT_IN(kern, lds);
   constexpr int bm = kWavesT * 16 * kQB;
