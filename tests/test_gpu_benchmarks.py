@@ -35,6 +35,23 @@ def test_mfma_ceiling_probe_runs_and_stays_under_the_peak():
         assert 500 < tflops < 2500 and 250 <= cycles < 400, out.stdout
 
 
+def test_simd_issue_probe_shows_what_the_attention_schedule_relies_on():
+    d = os.path.join(ROOT, "benchmarks", "cpp", "simd_issue")
+    path = os.path.join(d, "simd_issue")
+    if not os.path.exists(path):
+        subprocess.check_call(["make", "-C", d])
+    out = subprocess.run([path], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0 and out.stdout.rstrip().endswith("done"), out.stdout + out.stderr
+    rows = {line.split("|")[1]: [float(x) for x in line.split("|")[2:5]]
+            for line in out.stdout.splitlines() if line.startswith("|v_")}
+    # ordinary VALU instructions run at about half rate next to an MFMA stream; v_dot2 is far worse,
+    # which is why the attention kernel adds up its row sums on the matrix pipe
+    assert 4.0 < rows["v_fma_f32"][0] < 7.0 and 6.5 < rows["v_fma_f32"][1] < 11.0, out.stdout
+    assert rows["v_dot2c_f32_f16"][1] > 1.5 * rows["v_fma_f32"][1], out.stdout
+    blocks = [line.split("|") for line in out.stdout.splitlines() if line.startswith("|alone|") and line.count("|") == 4]
+    assert blocks and 1088 <= float(blocks[0][2]) < 2000 and 1088 <= float(blocks[0][3]) < 2000, out.stdout
+
+
 def test_fused_two_gemms_sweep_is_correct_on_a_few_shapes():
     import importlib.util
 
