@@ -50,6 +50,27 @@ def test_shapes(b, lq, lkv, d, causal, v_transposed):
     assert ok, f"rel_l2={r:.3e} max_abs={m:.3e}"
 
 
+# The 256-query workgroup keeps a five-tile ring with two tiles live and requests three tiles
+# ahead: key ranges of one to seven tiles, with and without a ragged last tile, exercise its fill,
+# the clamped requests past the end and the hand-over between the two wavefront sets; 768 queries
+# (an odd number of query tiles) take the one-pass causal order, 512 and 1024 the paired one.
+@pytest.mark.parametrize("lkv", [8, 64, 72, 128, 192, 200, 256, 320, 384, 448])
+@pytest.mark.parametrize("causal", [False, True])
+def test_short_key_ranges_through_the_eight_wavefront_ring(lkv, causal):
+    q, k, v = _inputs(2, 256, lkv, 128, 900 + lkv)
+    o = c_attention(q.to(DEV), k.to(DEV), v.to(DEV), causal, None, False)
+    ok, r, m = N.check_close(o, N.attention_ref(q, k, v, causal=causal))
+    assert ok, f"rel_l2={r:.3e} max_abs={m:.3e}"
+
+
+@pytest.mark.parametrize("lq,d", [(512, 128), (768, 128), (1024, 64), (300, 128)])
+def test_causal_pass_orders(lq, d):
+    q, k, v = _inputs(3, lq, lq, d, 77 + lq)
+    o = c_attention(q.to(DEV), k.to(DEV), v.to(DEV), True, None, False)
+    ok, r, m = N.check_close(o, N.attention_ref(q, k, v, causal=True))
+    assert ok, f"rel_l2={r:.3e} max_abs={m:.3e}"
+
+
 def test_scale_and_large_logits():
     # scale enters the logits; big logits need the running max (exp would overflow otherwise)
     q, k, v = _inputs(2, 128, 256, 128, 77)
