@@ -10,11 +10,12 @@
 //     flop sets its speed);
 //   * Q stays in registers for the whole workgroup (the reference reloads it per KV tile);
 //   * scores are computed transposed, S^T = K Q^T, so a lane owns one query row per 16-query
-//     block: its score values are plain registers, the running max / sum are in-lane
-//     reductions (the 4 lanes that share a query only talk when the reference max moves),
+//     block: its score values are plain registers, the running max is an in-lane
+//     reduction (the 4 lanes that share a query only talk when the reference max moves),
 //     and exp2(S^T) converted to fp16 is already the B-operand fragment of the second MFMA
 //     O^T = V^T P^T;
-//   * K and V tiles go global -> LDS directly (global_load_lds_dwordx4) into a 4-stage ring;
+//   * K and V tiles go global -> LDS directly (global_load_lds_dwordx4) into a ring of 5 tiles
+//     (4 for the 4-wavefront workgroup);
 //     V is kept [key][dim] in LDS and transposed on the way to registers with
 //     ds_read_b64_tr_b16; both tiles are XOR-swizzled against bank conflicts;
 //   * causal: tiles right of the diagonal are skipped, only tiles crossing it are masked.
