@@ -75,6 +75,24 @@ TF_API int tf_fused_two_gemms(const void* A, const void* B, const void* C, void*
                               int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P, int tm,
                               int tn, int tk, int tp, void* stream);
 
+/* tf_fused_two_gemms with a caller-provided device workspace.  Long-N fp16 problems (K = P = 128, N
+ * a multiple of 64, too few row blocks to fill the chip) are then cut along N wherever that is the
+ * faster way: each workgroup takes a range of N for its rows, fp32 partial results go to the
+ * workspace and a second kernel adds them up into D.  tf_fused_two_gemms_workspace_bytes says how many bytes that takes
+ * for a problem (0: it would not be cut); with a null or smaller workspace, and for every other
+ * shape or type, tf_fused_two_gemms_ws is tf_fused_two_gemms.  The workspace must be 16-byte
+ * aligned; its contents are scratch.  Results equal those of tf_fused_two_gemms up to the order of
+ * the fp32 additions over N.
+ * No counterpart in the reference, whose op has no workspace (src/kernels/fused_two_gemms.cu:66-144
+ * launches M / tm x P / tp blocks that each walk all of N); the torch op of this library allocates
+ * the workspace itself, so callers of the reference's Python / torch API get the cut for free. */
+TF_API size_t tf_fused_two_gemms_workspace_bytes(int dtype, int64_t batch, int64_t M, int64_t N,
+                                                 int64_t K, int64_t P);
+TF_API int tf_fused_two_gemms_ws(const void* A, const void* B, const void* C, void* D, int dtype,
+                                 int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P, int tm,
+                                 int tn, int tk, int tp, void* workspace, size_t workspace_bytes,
+                                 void* stream);
+
 /* O = softmax(scale * Q K^T (+ causal mask)) V for `batch` independent (batch x head)
  * slices laid out back to back.  fp16 in/out, fp32 scores, fp32 running max / sum.
  * Q [batch, Lq, D]; K [batch, Lkv, D]; V [batch, Lkv, Dv] when v_is_transposed == 0, or

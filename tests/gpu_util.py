@@ -36,6 +36,24 @@ def c_fused(a, b, c, tiles=None):
     return d
 
 
+def c_fused_ws(a, b, c, tiles=None, workspace_bytes=None):
+    """The workspace form: returns (D, bytes the library asked for).  workspace_bytes overrides the
+    size that is handed over (0: no workspace)."""
+    lib = _capi.load()
+    batch = 1 if a.dim() == 2 else a.shape[0]
+    m, k = a.shape[-2:]
+    n, p = b.shape[-2], c.shape[-2]
+    tm, tn, tk, tp = tiles if tiles else (m, n, k, p)
+    want = lib.tf_fused_two_gemms_workspace_bytes(_capi.TF_DTYPE_F16, batch, m, n, k, p)
+    nbytes = want if workspace_bytes is None else workspace_bytes
+    ws = torch.full((max(nbytes, 16),), 0xFF, device=a.device, dtype=torch.uint8)
+    d = torch.full((*a.shape[:-1], p), float("nan"), device=a.device, dtype=torch.float16)
+    _capi.check(lib.tf_fused_two_gemms_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), _capi.TF_DTYPE_F16,
+                                          batch, m, n, k, p, tm, tn, tk, tp, ws.data_ptr() if nbytes else None,
+                                          nbytes, stream()), "tf_fused_two_gemms_ws")
+    return d, want
+
+
 def c_attention(q, k, v, causal=False, scale=None, v_transposed=False, tiles=None):
     """q [B, Lq, D], k [B, Lkv, D], v [B, Lkv, Dv] (or [B, Dv, Lkv] if v_transposed)."""
     lib = _capi.load()

@@ -6,7 +6,7 @@ import torch
 
 import oracle
 from oracle import numerics as N
-from tests.gpu_util import DEV, c_fused
+from tests.gpu_util import DEV, c_fused, c_fused_ws
 
 pytestmark = pytest.mark.gpu
 
@@ -58,6 +58,45 @@ def test_streaming_kernel_exact(batch, m, n):
     for i in range(batch):
         ref = N.fused_two_gemms_ref_rounded(a[i], b[i], c[i])
         assert torch.equal(d[i].float(), ref.half().float()), f"batch {i}"
+
+
+# With a workspace the long-N problems are cut along N (fp32 partial sums per part, added up by a
+# second kernel).  The same exact-integer construction: the cut result must equal the oracle and the
+# uncut kernel bit for bit.  Shapes: parts of equal and of unequal length, a ragged last row block,
+# a batch, one row (all with 64-row blocks, four wavefronts x two sets); 4096 and 4000 rows x 4096
+# take 128-row blocks (eight wavefronts, every one on every tile), the second with a ragged block.
+@pytest.mark.parametrize("batch,m,n", [(1, 64, 2048), (1, 70, 1856), (1, 1, 2048), (1, 200, 2112), (3, 96, 1600),
+                                       (1, 4096, 2048), (1, 4096, 4096), (1, 4000, 4096)])
+def test_split_along_n_is_exact(batch, m, n):
+    g = torch.Generator().manual_seed(19 * m + n + batch)
+    a = torch.randint(-2, 3, (batch, m, 128), generator=g).half()
+    b = (torch.randint(-2, 3, (batch, n, 128), generator=g) / 4).half()
+    c = (torch.randint(-2, 3, (batch, 128, n), generator=g) / 8).half()
+    ad, bd, cd = a.to(DEV), b.to(DEV), c.to(DEV)
+    d, want = c_fused_ws(ad, bd, cd)
+    assert want > 0 and want % (batch * m * 128 * 4) == 0
+    assert torch.equal(d, c_fused(ad, bd, cd))
+    d = d.cpu()
+    for i in range(batch if m <= 200 else 0):
+        ref = N.fused_two_gemms_ref_rounded(a[i], b[i], c[i])
+        assert torch.equal(d[i].float(), ref.half().float()), f"batch {i}"
+
+
+def test_workspace_form_without_a_cut_is_the_plain_op():
+    g = torch.Generator().manual_seed(5)
+    a = (torch.randn(300 * 64, 128, generator=g) / 8).half().to(DEV)
+    b = (torch.randn(2048, 128, generator=g) / 8).half().to(DEV)
+    c = (torch.randn(128, 2048, generator=g) / 8).half().to(DEV)
+    d, want = c_fused_ws(a, b, c)
+    assert want == 0 and torch.equal(d, c_fused(a, b, c))          # enough row blocks: not cut
+    d, want = c_fused_ws(a[:64], b[:512].contiguous(), c[:, :512].contiguous())
+    assert want == 0                                               # eight n-tiles: a cut would not pay
+    a = a[:4096].contiguous()
+    d, want = c_fused_ws(a, b, c, workspace_bytes=0)               # no workspace handed over: not cut
+    assert want > 0 and torch.equal(d, c_fused(a, b, c))
+    d2, _ = c_fused_ws(a, b, c)                                    # cut: same sums in another order
+    ok, r, m = N.check_close(d2, d.float().cpu())
+    assert ok and r < 1e-3
 
 
 def test_batched():

@@ -22,6 +22,8 @@ SIGNATURES = {
     "tf_flash_attention_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _i, _d, _i, _vp]),
     "tf_gemm": (_i, [_vp, _vp, _vp, _i, _i, _i64, _i64, _i64, _i, _i, _i, _i, _i, _vp]),
     "tf_fused_two_gemms": (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _vp]),
+    "tf_fused_two_gemms_workspace_bytes": (_sz, [_i, _i64, _i64, _i64, _i64, _i64]),
+    "tf_fused_two_gemms_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _vp, _sz, _vp]),
     "tf_flash_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i64, _i64, _i64, _i64, _i64, _i, _i, _i, _i, _i, _d, _i, _vp]),
     "tf_flash_decode_workspace_bytes": (_sz, [_i64, _i64, _i]),
     "tf_flash_decode_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i, _d, _vp]),

@@ -14,6 +14,8 @@
 //     tiles shared by the 4 wavefronts; A fragments are private to a wavefront and are read
 //     straight from global memory into registers;
 //   * D is staged through LDS so that global stores are 16 bytes per lane along rows.
+#include <algorithm>
+
 #include "common.hpp"
 #include "jit_ops.hpp"
 
@@ -376,18 +378,24 @@ int launch(const void* A, const void* B, const void* C, void* D, int batch, int 
 // end.  A wavefront's chain per tile - fragment reads, 16 MFMAs, fp16 conversion, 16 MFMAs that
 // depend on it - leaves the matrix pipe idle most of the time; a second, independent chain on
 // the same SIMD fills it.  Only the first set issues the tile requests.
-template <int kWavesT, int kSplit>
+// kPartial: blockIdx.y selects a part of `tiles_per_part` n-tiles, and the workgroup writes its fp32
+// partial sums to part blockIdx.y of the workspace W [batch][parts][M][128] instead of D; a second
+// kernel adds the parts up.  M / 64 workgroups do not fill the chip for the shapes this kernel is
+// for, and a workgroup is bound by how many tile bytes its ring keeps in flight, not by arithmetic.
+template <int kWavesT, int kSplit, bool kPartial>
 __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_kernel(
     const half_t* __restrict__ A, const half_t* __restrict__ B, const half_t* __restrict__ C,
-    half_t* __restrict__ D, int M, int N) {
+    half_t* __restrict__ D, float* __restrict__ W, int M, int N, int tiles_per_part) {
   constexpr int K = 128, P = 128, TN = 64, kStagesS = 4;
   constexpr int kRows = 16 * kWavesT;
   constexpr int kBBytes = TN * K * 2;                // 16 KiB: B tile [n][k], 256-byte rows
   constexpr int kCBytes = P * TN * 2;                // 16 KiB: C tile [p][n], 128-byte rows
   constexpr int kStageBytes = kBBytes + kCBytes;
   constexpr int kBInstr = kBBytes / 1024, kCInstr = kCBytes / 1024;   // 1 KiB wavefront requests
-  constexpr int kReqPerWave = (kBInstr + kCInstr) / kWavesT;
-  static_assert((kBInstr / kWavesT) % 4 == 0 && (kCInstr / kWavesT) % 4 == 0,
+  // the first kReqWaves wavefronts issue the tile requests (all of them when there are four)
+  constexpr int kReqWaves = kWavesT > 4 ? 4 : kWavesT;
+  constexpr int kReqPerWave = (kBInstr + kCInstr) / kReqWaves;
+  static_assert((kBInstr / kReqWaves) % 4 == 0 && (kCInstr / kReqWaves) % 4 == 0,
                 "a wavefront's requests of a tile come in groups of four consecutive instructions");
   // tiles requested ahead of the one being multiplied: the ring allows kStagesS - 1, the 6-bit
   // vmcnt allows 63 requests of one wavefront to stay in flight behind the awaited tile
@@ -413,7 +421,9 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
   for (int ks = 0; ks < 4; ++ks)
     af[ks] = *reinterpret_cast<const half8_t*>(A + (size_t)a_row * K + 8 * lg + ks * 32);
 
-  const int n_tiles = N / TN;
+  // this workgroup's n-tiles: [t_begin, t_begin + n_tiles)
+  const int t_begin = kPartial ? (int)blockIdx.y * tiles_per_part : 0;
+  const int n_tiles = kPartial ? min(tiles_per_part, N / TN - t_begin) : N / TN;
   // Requests of n-tile t (clamped past the end: the surplus lands in a stage nobody reads
   // again).  Instruction i of the B tile covers rows 4i .. 4i+3 (16 chunks each), of the C tile
   // rows 8i .. 8i+7 (8 chunks each); lane l fills physical chunk l % 16 (l % 8) and fetches the
@@ -424,15 +434,15 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
   const unsigned voff_b0 = (lane / 16) * (K * 2) + (((lane % 16) ^ (lane / 16)) << 4);
   const unsigned voff_c0 = (lane / 8) * (unsigned)N * 2u + (((lane % 8) ^ (lane / 16)) << 4);
   auto request_tile = [&](int t) __attribute__((always_inline)) {
-    if (kSplit > 1 && half != 0) return;
+    if (wave_id >= kReqWaves) return;
     const unsigned stage = smem_base + (t % kStagesS) * kStageBytes;
-    const int n0 = min(t, n_tiles - 1) * TN;
+    const int n0 = (t_begin + min(t, n_tiles - 1)) * TN;
     const char* b_src = reinterpret_cast<const char*>(B) + (size_t)n0 * (K * 2);
     const char* c_src = reinterpret_cast<const char*>(C) + (size_t)n0 * 2;
 #pragma unroll
-    for (int q = 0; q < kBInstr / kWavesT; ++q) {
-      // instructions are dealt in blocks of kBInstr / kWavesT consecutive ones per wavefront
-      const int i_first = wave * (kBInstr / kWavesT);
+    for (int q = 0; q < kBInstr / kReqWaves; ++q) {
+      // instructions are dealt in blocks of kBInstr / kReqWaves consecutive ones per wavefront
+      const int i_first = wave_id * (kBInstr / kReqWaves);
       const unsigned voff = voff_b0 ^ (unsigned)(((q % 4) * 4) << 4);        // row 4i: chunk ^= 4 * (i % 4)
       const char* src = b_src + (size_t)(i_first + q) * 1024 - (q % 4) * 1024;   // + rows, - what the immediate adds
       if (q % 4 == 0)
@@ -441,8 +451,8 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
         asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(src), "n"(1024 * (q % 4)) : "memory");
     }
 #pragma unroll
-    for (int q = 0; q < kCInstr / kWavesT; ++q) {
-      const int i_first = wave * (kCInstr / kWavesT);
+    for (int q = 0; q < kCInstr / kReqWaves; ++q) {
+      const int i_first = wave_id * (kCInstr / kReqWaves);
       const unsigned voff = voff_c0 ^ (unsigned)(((q % 2) * 4) << 4);        // row 8i: chunk ^= 4 * (i % 2)
       const char* src = c_src + (size_t)(i_first + q) * 8 * (size_t)N * 2 - (q % 4) * 1024;
       if (q % 4 == 0)
@@ -496,8 +506,21 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
     }
   }
 
-  // Epilogue: acc2[pt][r] = D[m0 + 16*wave + 4*lg + r][16*pt + lr], staged through LDS for
-  // 16-byte stores along rows
+  // Epilogue: acc2[pt][r] = D[m0 + 16*wave + 4*lg + r][16*pt + lr]
+  if constexpr (kPartial) {
+    // fp32 partial sums straight from the accumulators: 16 adjacent lanes write 64 contiguous bytes
+    if (half == 0) {
+      float* w = W + ((batch * gridDim.y + blockIdx.y) * (size_t)M + m0 + wave * 16 + 4 * lg) * P + lr;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (m0 + wave * 16 + 4 * lg + r < M) {
+#pragma unroll
+          for (int pt = 0; pt < 8; ++pt) __builtin_nontemporal_store(acc2[pt][r], w + (size_t)r * P + pt * 16);
+        }
+    }
+    return;
+  }
+  // fp16 result, staged through LDS for 16-byte stores along rows
   if (half == 0) {
 #pragma unroll
     for (int pt = 0; pt < 8; ++pt)
@@ -514,17 +537,82 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
   }
 }
 
+// D[b][i] = fp16(sum over parts of W[b][part][i]), i over the M * 128 elements of a problem
+__global__ __launch_bounds__(256) void fused_two_gemms_reduce_kernel(const float* __restrict__ W,
+                                                                     half_t* __restrict__ D, int parts,
+                                                                     size_t elems) {
+  const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= elems) return;
+  const float* w = W + (size_t)blockIdx.z * parts * elems + i;
+  float4_t acc = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(w));
+  for (int part = 1; part < parts; ++part)
+    acc += __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(w + (size_t)part * elems));
+  half4_t h = {(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
+  *reinterpret_cast<half4_t*>(D + (size_t)blockIdx.z * elems + i) = h;
+}
+
 template <int kWavesT, int kSplit>
 int launch_stream(const void* A, const void* B, const void* C, void* D, int batch, int M, int N,
                   hipStream_t st) {
-  auto kern = fused_two_gemms_stream_kernel<kWavesT, kSplit>;
+  auto kern = fused_two_gemms_stream_kernel<kWavesT, kSplit, false>;
   constexpr int lds = 4 * (64 * 128 * 2 + 128 * 64 * 2) + 16 * kWavesT * 128 * 2;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
   TFK_LDS_OPT_IN(kern, lds);
   dim3 grid((M + 16 * kWavesT - 1) / (16 * kWavesT), 1, batch);
   hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const half_t*>(A),
                      static_cast<const half_t*>(B), static_cast<const half_t*>(C),
-                     static_cast<half_t*>(D), M, N);
+                     static_cast<half_t*>(D), static_cast<float*>(nullptr), M, N, 0);
+  TFK_HIP_TRY(hipGetLastError());
+  return TF_OK;
+}
+
+// How a long-N problem (K = P = 128) is cut when a workspace is available: `parts` ranges of
+// `tiles_per_part` 64-wide n-tiles for row blocks of `rows` rows.  A workgroup takes a CU to itself
+// (the ring fills its LDS) and is bound by the tile bytes it keeps in flight, so the cut aims at one
+// workgroup per CU (row blocks x parts <= 256) and keeps at least the four tiles per part that
+// fill the ring.  Measured on the reference's sweep, a launch takes about 9.6 + 0.9 t us with
+// 64-row blocks and 11.8 + 1.23 t us with 128-row blocks (eight wavefronts share every tile), t the
+// tiles a workgroup walks, against 4 + 0.8 t uncut: the second launch and the trip of the partial
+// sums through memory are in the constants.  The cheapest of the three is taken; 128-row blocks
+// only from eight tiles per part on (shorter walks are dominated by filling the ring, and eight
+// wavefronts fill it no faster than four).  parts == 1: no cut.
+struct SplitPlan { int parts, tiles_per_part, rows; };
+SplitPlan fused_split_plan(int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P) {
+  const SplitPlan uncut = {1, 0, 64};
+  if (!(K == 128 && P == 128 && N % 64 == 0 && N >= 512)) return uncut;
+  const int64_t n_tiles = N / 64;
+  auto cut = [&](int rows) -> SplitPlan {
+    const int64_t row_blocks = (M + rows - 1) / rows * batch;
+    int64_t parts = std::min<int64_t>(256 / std::max<int64_t>(row_blocks, 1), n_tiles / 4);
+    if (parts <= 1) return {1, 0, rows};
+    const int64_t per = (n_tiles + parts - 1) / parts;
+    return {(int)((n_tiles + per - 1) / per), (int)per, rows};
+  };
+  const SplitPlan p64 = cut(64), p128 = cut(128);
+  double best = 4.0 + 0.8 * (double)n_tiles;
+  SplitPlan plan = uncut;
+  if (p64.parts > 1 && 9.6 + 0.9 * p64.tiles_per_part < best) {
+    best = 9.6 + 0.9 * p64.tiles_per_part;
+    plan = p64;
+  }
+  if (p128.parts > 1 && p128.tiles_per_part >= 8 && 11.8 + 1.23 * p128.tiles_per_part < best) plan = p128;
+  return plan;
+}
+
+template <int kWavesT, int kSplit>
+int launch_stream_split(const void* A, const void* B, const void* C, void* D, float* W, SplitPlan plan, int batch,
+                        int M, int N, hipStream_t st) {
+  auto kern = fused_two_gemms_stream_kernel<kWavesT, kSplit, true>;
+  constexpr int lds = 4 * (64 * 128 * 2 + 128 * 64 * 2) + 16 * kWavesT * 128 * 2;
+  TFK_LDS_OPT_IN(kern, lds);
+  dim3 grid((M + 16 * kWavesT - 1) / (16 * kWavesT), plan.parts, batch);
+  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const half_t*>(A),
+                     static_cast<const half_t*>(B), static_cast<const half_t*>(C),
+                     static_cast<half_t*>(D), W, M, N, plan.tiles_per_part);
+  TFK_HIP_TRY(hipGetLastError());
+  const size_t elems = (size_t)M * 128;
+  hipLaunchKernelGGL(fused_two_gemms_reduce_kernel, dim3((unsigned)((elems / 4 + 255) / 256), 1, batch), dim3(256), 0,
+                     st, W, static_cast<half_t*>(D), plan.parts, elems);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
 }
@@ -579,6 +667,32 @@ extern "C" int tf_fused_two_gemms_f16(const void* A, const void* B, const void* 
     return launch_stream<4, 2>(A, B, C, D, (int)batch, (int)M, (int)N, st);
   if (N % 128 == 0) return pick_tp<128>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
   return pick_tp<32>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
+}
+
+extern "C" size_t tf_fused_two_gemms_workspace_bytes(int dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                                                     int64_t P) {
+  using namespace tfk;
+  if (dtype != TF_DTYPE_F16 || batch <= 0 || M <= 0 || N <= 0) return 0;
+  const SplitPlan plan = fused_split_plan(batch, M, N, K, P);
+  return plan.parts > 1 ? (size_t)plan.parts * (size_t)batch * (size_t)M * 128 * sizeof(float) : 0;
+}
+
+extern "C" int tf_fused_two_gemms_ws(const void* A, const void* B, const void* C, void* D, int dtype, int64_t batch,
+                                     int64_t M, int64_t N, int64_t K, int64_t P, int tm, int tn, int tk, int tp,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+  using namespace tfk;
+  const size_t want = tf_fused_two_gemms_workspace_bytes(dtype, batch, M, N, K, P);
+  if (want == 0 || workspace == nullptr || workspace_bytes < want)
+    return tf_fused_two_gemms(A, B, C, D, dtype, batch, M, N, K, P, tm, tn, tk, tp, stream);
+  if (int rc = check_fused_args("tf_fused_two_gemms_ws", A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp)) return rc;
+  TFK_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, TF_ERR_INVALID_ARG,
+              "tf_fused_two_gemms_ws: workspace must be 16-byte aligned");
+  const SplitPlan plan = fused_split_plan(batch, M, N, K, P);
+  if (plan.rows == 128)
+    return launch_stream_split<8, 1>(A, B, C, D, static_cast<float*>(workspace), plan, (int)batch, (int)M, (int)N,
+                                     static_cast<hipStream_t>(stream));
+  return launch_stream_split<4, 2>(A, B, C, D, static_cast<float*>(workspace), plan,
+                                   (int)batch, (int)M, (int)N, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tf_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype, int64_t batch,

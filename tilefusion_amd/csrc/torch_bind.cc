@@ -123,8 +123,13 @@ void fused_two_gemms(const at::Tensor& A, const at::Tensor& B, const at::Tensor&
   const int64_t kp = round_up(k, 32), np = round_up(n, 32), pp = round_up(p, 16);
   const int64_t mp = dtype == TF_DTYPE_BF16 ? round_up(m, 16) : m;
   if (kp == k && np == n && pp == p && mp == m) {
-    check_status(tf_fused_two_gemms(A.data_ptr(), B.data_ptr(), C.data_ptr(), D.data_ptr(), dtype, batch,
-                                    m, n, k, p, (int)tm, (int)tn, (int)tk, (int)tp, current_stream()),
+    // long-N problems are cut along N when the library is handed a workspace for the partial sums
+    const size_t ws_bytes = tf_fused_two_gemms_workspace_bytes(dtype, batch, m, n, k, p);
+    at::Tensor ws;
+    if (ws_bytes > 0) ws = at::empty({(int64_t)ws_bytes}, A.options().dtype(at::kByte));
+    check_status(tf_fused_two_gemms_ws(A.data_ptr(), B.data_ptr(), C.data_ptr(), D.data_ptr(), dtype, batch,
+                                       m, n, k, p, (int)tm, (int)tn, (int)tk, (int)tp,
+                                       ws_bytes > 0 ? ws.data_ptr() : nullptr, ws_bytes, current_stream()),
                  "fused_two_gemms");
     return;
   }
