@@ -82,6 +82,22 @@ def test_split_along_n_is_exact(batch, m, n):
         assert torch.equal(d[i].float(), ref.half().float()), f"batch {i}"
 
 
+def test_many_rows_take_128_row_blocks_exactly():
+    # 256 blocks of 128 rows and more run eight wavefronts on every tile; the last block is ragged
+    g = torch.Generator().manual_seed(23)
+    m, n = 256 * 128 + 40, 576
+    a = torch.randint(-2, 3, (m, 128), generator=g).half()
+    b = (torch.randint(-2, 3, (n, 128), generator=g) / 4).half()
+    c = (torch.randint(-2, 3, (128, n), generator=g) / 8).half()
+    d = c_fused(a.to(DEV), b.to(DEV), c.to(DEV)).cpu()
+    for rows in (slice(0, 300), slice(m - 300, m)):
+        ref = N.fused_two_gemms_ref_rounded(a[rows], b, c)
+        assert torch.equal(d[rows].float(), ref.half().float())
+    # every row block agrees with the 64-row kernel, which a shorter problem runs
+    d_small = c_fused(a[:8192].to(DEV), b.to(DEV), c.to(DEV)).cpu()
+    assert torch.equal(d[:8192], d_small)
+
+
 def test_workspace_form_without_a_cut_is_the_plain_op():
     g = torch.Generator().manual_seed(5)
     a = (torch.randn(300 * 64, 128, generator=g) / 8).half().to(DEV)
