@@ -1,7 +1,8 @@
 """Flash-attention forward over head dimensions: the tuned kernels (D = 64, 128; fp16 and bf16)
 next to the header macro kernel ke_flash_attention compiled at run time (what any other head
 dimension runs, here D = 96 and D = 32), all through the same entry point
-tf_flash_attention_fwd.  Counterpart of the reference's benchmarks/cpp/flashattention
+tf_flash_attention_fwd; and the torch op for those head dimensions, which zero-pads them to the
+next tuned size instead (TFLOP/s count the unpadded problem).  Counterpart of the reference's benchmarks/cpp/flashattention
 program; every row is checked against an fp32 softmax(QK^T)V of one (batch, head) slice.
 
     python benchmarks/attention/bench.py      # prints a markdown table
@@ -21,7 +22,9 @@ BH, S = 32, 4096
 CASES = [(128, torch.float16, False, "tuned"), (128, torch.float16, True, "tuned"), (128, torch.bfloat16, False, "tuned"),
          (64, torch.float16, False, "tuned"), (96, torch.float16, False, "header kernel"),
          (96, torch.float16, True, "header kernel"), (96, torch.bfloat16, False, "header kernel"),
-         (32, torch.float16, False, "header kernel")]
+         (32, torch.float16, False, "header kernel"),
+         (96, torch.float16, False, "torch op: padded to 128, tuned"), (96, torch.float16, True, "torch op: padded to 128, tuned"),
+         (32, torch.float16, False, "torch op: padded to 64, tuned")]
 
 
 def _time_ms(fn, warm=60, reps=40):
@@ -51,7 +54,12 @@ def run(cases=CASES, bh=BH, s=S, out=sys.stdout):
         code = _capi.TF_DTYPE_BF16 if dtype == torch.bfloat16 else _capi.TF_DTYPE_F16
         st = torch.cuda.current_stream().cuda_stream
 
+        def call_op():
+            torch.ops.tilefusion.flash_attention(q, k, vt, o, 64, 64, d, d, scale, causal)
+
         def call():
+            if what.startswith("torch op"):
+                return call_op()
             rc = lib.tf_flash_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), o.data_ptr(), code, bh, s, s, d, d,
                                             1, 64, 64, d, d, scale, int(causal), st)
             assert rc == 0, lib.tf_last_error()

@@ -107,10 +107,12 @@ def _close_bf16(out, ref):
 
 
 @pytest.mark.parametrize("d,dv,lq,lkv,causal", [(64, 128, 128, 256, False), (96, 96, 128, 128, True),
-                                                (48, 80, 64, 128, False), (128, 64, 40, 64, True)])
+                                                (48, 80, 64, 128, False), (128, 64, 40, 64, True),
+                                                (48, 48, 200, 160, True), (32, 16, 64, 96, False)])
 def test_flash_attention_ops_for_head_dims_without_a_tuned_kernel(d, dv, lq, lkv, causal):
-    # (64, 128), (96, 96): run-time compiled from the header kernel as they are; (48, 80): zero-padded
-    # to (64, 80); Lq = 40: padded to 48 query rows.  Both op forms (natural and transposed V).
+    # Head dimensions up to 128 without a tuned kernel are zero-padded by the op to the next tuned
+    # size ((48, 48) -> 64, the others -> 128) and run the tuned kernel, any Lq and Lkv.  Both op
+    # forms (natural and transposed V).
     from tilefusion_amd.ops import flash_attention
     g = torch.Generator().manual_seed(d * 1000 + dv)
     q = torch.randn(2, lq, d, generator=g).half()
@@ -129,11 +131,27 @@ def test_flash_attention_ops_for_head_dims_without_a_tuned_kernel(d, dv, lq, lkv
     assert ok, (r, m)
 
 
+@pytest.mark.parametrize("d,dv,lq,lkv", [(160, 160, 48, 64), (192, 128, 40, 96)])
+def test_flash_attention_ops_for_head_dims_above_128_run_the_header_kernel(d, dv, lq, lkv):
+    # no tuned kernel and nothing to pad to: compiled at run time from the header kernel (query rows
+    # padded to whole MFMA tiles by the op)
+    g = torch.Generator().manual_seed(d + dv)
+    q = torch.randn(1, lq, d, generator=g).half()
+    k = torch.randn(1, lkv, d, generator=g).half()
+    v = torch.randn(1, lkv, dv, generator=g).half()
+    scale = 1.0 / math.sqrt(d)
+    o = torch.full((1, lq, dv), float("nan"), dtype=torch.float16, device=DEV)
+    torch.ops.tilefusion.flash_attention_fwd(q.to(DEV), k.to(DEV), v.to(DEV), o, scale, False)
+    ok, r, m = N.check_close(o, N.attention_ref(q, k, v, scale, False))
+    assert ok, (r, m)
+
+
 def test_flash_attention_key_length_that_cannot_be_padded_is_a_clear_error():
-    q = torch.randn(16, 96, dtype=torch.float16, device=DEV)
-    k = torch.randn(48, 96, dtype=torch.float16, device=DEV)
-    v = torch.randn(48, 96, dtype=torch.float16, device=DEV)
-    o = torch.zeros(16, 96, dtype=torch.float16, device=DEV)
+    # above 128 the header kernel is what runs, and its key tiles are 32 wide
+    q = torch.randn(16, 160, dtype=torch.float16, device=DEV)
+    k = torch.randn(48, 160, dtype=torch.float16, device=DEV)
+    v = torch.randn(48, 160, dtype=torch.float16, device=DEV)
+    o = torch.zeros(16, 160, dtype=torch.float16, device=DEV)
     with pytest.raises(RuntimeError, match="multiple of 32"):
         torch.ops.tilefusion.flash_attention_fwd(q, k, v, o, 0.1, False)
 
