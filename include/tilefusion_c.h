@@ -69,16 +69,16 @@ TF_API int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, v
                                   int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P,
                                   int tm, int tn, int tk, int tp, void* stream);
 
-/* The same for fp16 or bf16 (dtype as in tf_gemm); bf16 is compiled at run time from the header
- * kernel (M multiple of 16, N and K of 32, P of 16). */
+/* The same for fp16 or bf16 (dtype as in tf_gemm): the same kernels with the bf16 MFMA, a bf16
+ * intermediate and bf16 output. */
 TF_API int tf_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype,
                               int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P, int tm,
                               int tn, int tk, int tp, void* stream);
 
-/* tf_fused_two_gemms with a caller-provided device workspace.  Long-N fp16 problems (K = P = 128, N
+/* tf_fused_two_gemms with a caller-provided device workspace.  Long-N problems (K = P = 128, N
  * a multiple of 64, too few row blocks to fill the chip) are then cut along N wherever that is the
  * faster way: each workgroup takes a range of N for its rows, fp32 partial results go to the
- * workspace and a second kernel adds them up into D.  tf_fused_two_gemms_workspace_bytes says how many bytes that takes
+ * workspace and a second kernel adds them up into D (fp16 and bf16).  tf_fused_two_gemms_workspace_bytes says how many bytes that takes
  * for a problem (0: it would not be cut); with a null or smaller workspace, and for every other
  * shape or type, tf_fused_two_gemms_ws is tf_fused_two_gemms.  The workspace must be 16-byte
  * aligned; its contents are scratch.  Results equal those of tf_fused_two_gemms up to the order of

@@ -36,6 +36,26 @@ def c_fused(a, b, c, tiles=None):
     return d
 
 
+def c_fused_dtype(a, b, c, tiles=None, workspace=False):
+    """The dtype-coded entry points (fp16 or bf16 operands), without or with a workspace."""
+    lib = _capi.load()
+    batch = 1 if a.dim() == 2 else a.shape[0]
+    m, k = a.shape[-2:]
+    n, p = b.shape[-2], c.shape[-2]
+    tm, tn, tk, tp = tiles if tiles else (m, n, k, p)
+    code = _capi.TF_DTYPE_BF16 if a.dtype == torch.bfloat16 else _capi.TF_DTYPE_F16
+    d = torch.full((*a.shape[:-1], p), float("nan"), device=a.device, dtype=a.dtype)
+    if not workspace:
+        _capi.check(lib.tf_fused_two_gemms(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), code, batch,
+                                           m, n, k, p, tm, tn, tk, tp, stream()), "tf_fused_two_gemms")
+        return d
+    want = lib.tf_fused_two_gemms_workspace_bytes(code, batch, m, n, k, p)
+    ws = torch.empty(max(want, 16), device=a.device, dtype=torch.uint8)
+    _capi.check(lib.tf_fused_two_gemms_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), d.data_ptr(), code, batch, m, n, k, p,
+                                          tm, tn, tk, tp, ws.data_ptr(), want, stream()), "tf_fused_two_gemms_ws")
+    return d
+
+
 def c_fused_ws(a, b, c, tiles=None, workspace_bytes=None):
     """The workspace form: returns (D, bytes the library asked for).  workspace_bytes overrides the
     size that is handed over (0: no workspace)."""

@@ -6,7 +6,7 @@ import torch
 
 import oracle
 from oracle import numerics as N
-from tests.gpu_util import DEV, c_fused, c_fused_ws
+from tests.gpu_util import DEV, c_fused, c_fused_dtype, c_fused_ws
 
 pytestmark = pytest.mark.gpu
 
@@ -113,6 +113,37 @@ def test_workspace_form_without_a_cut_is_the_plain_op():
     d2, _ = c_fused_ws(a, b, c)                                    # cut: same sums in another order
     ok, r, m = N.check_close(d2, d.float().cpu())
     assert ok and r < 1e-3
+
+
+# bf16 runs the same kernels with the bf16 MFMA.  Small integers are exact in bf16 too, so the plain
+# kernel (one n-tile, several n-tiles, ragged rows), the streaming kernel and the cut along N are
+# compared bit for bit with the oracle evaluated on the same values; a random case bounds the error
+# of the bf16 rounding of the intermediate (8 mantissa bits): rel-L2 <= 4e-3.
+@pytest.mark.parametrize("m,n,k,p,workspace", [(256, 128, 128, 128, False), (70, 96, 64, 48, False), (130, 384, 128, 128, False),
+                                               (64, 2048, 128, 128, True), (4096, 4096, 128, 128, True)])
+def test_bf16_kernels_exact(m, n, k, p, workspace):
+    g = torch.Generator().manual_seed(m + n + k + p)
+    a = torch.randint(-2, 3, (m, k), generator=g).bfloat16()
+    b = (torch.randint(-2, 3, (n, k), generator=g) / 4).bfloat16()
+    c = (torch.randint(-2, 3, (p, n), generator=g) / 8).bfloat16()
+    d = c_fused_dtype(a.to(DEV), b.to(DEV), c.to(DEV), workspace=workspace).cpu()
+    rows = slice(0, min(m, 256))
+    inter = (a[rows].float() @ b.float().T)
+    assert torch.equal(inter.bfloat16().float(), inter)            # the intermediate is exact in bf16
+    ref = inter @ c.float().T
+    assert torch.equal(d[rows].float(), ref.bfloat16().float())
+    if workspace:
+        assert torch.equal(d, c_fused_dtype(a.to(DEV), b.to(DEV), c.to(DEV)).cpu())
+
+
+def test_bf16_random_inputs_within_tolerance():
+    g = torch.Generator().manual_seed(77)
+    a = (torch.randn(512, 128, generator=g) / 11).bfloat16()
+    b = (torch.randn(128, 128, generator=g) / 11).bfloat16()
+    c = (torch.randn(128, 128, generator=g) / 11).bfloat16()
+    d = c_fused_dtype(a.to(DEV), b.to(DEV), c.to(DEV))
+    ref = N.fused_two_gemms_ref(a, b, c)
+    assert N.rel_l2(d, ref) <= 4e-3 and N.max_abs(d, ref) <= 4e-2 * max(1.0, float(ref.abs().max()))
 
 
 def test_batched():

@@ -1,6 +1,6 @@
-// Fused back-to-back GEMM for gfx950: D[M,P] = (A[M,K] * B[K,N]) * C[N,P], fp16 in/out, fp32
-// accumulate; the intermediate A*B lives only in registers (rounded to fp16 like the
-// reference does, include/kernels/fused_two_gemms_device.cuh:200).
+// Fused back-to-back GEMM for gfx950: D[M,P] = (A[M,K] * B[K,N]) * C[N,P], fp16 or bf16 in/out,
+// fp32 accumulate; the intermediate A*B lives only in registers (rounded to the element type like
+// the reference does, include/kernels/fused_two_gemms_device.cuh:200).
 //
 // Counterpart of ke_fused_two_gemms (include/kernels/fused_two_gemms_device.cuh:114-214) and its
 // host launcher (src/kernels/fused_two_gemms.cu:66-144).  CDNA4 design:
@@ -15,12 +15,23 @@
 //     straight from global memory into registers;
 //   * D is staged through LDS so that global stores are 16 bytes per lane along rows.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.hpp"
-#include "jit_ops.hpp"
 
 namespace tfk {
 namespace {
+
+// The kernels move 16-bit elements without looking at them; the element type T (half_t or bf16_t)
+// only selects the MFMA and the float -> T conversions.
+template <typename T> using vec2_t = T __attribute__((ext_vector_type(2)));
+template <typename T> using vec4_t = T __attribute__((ext_vector_type(4)));
+template <typename T> using vec8_t = T __attribute__((ext_vector_type(8)));
+template <typename T>
+TFK_DEVICE float4_t mfma_t(vec8_t<T> a, vec8_t<T> b, float4_t c) {
+  if constexpr (std::is_same_v<T, bf16_t>) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  else return mfma_16x16x32(a, b, c);
+}
 
 constexpr int kRowsPerBlock = 64;
 constexpr int kWaves = 4;
@@ -35,8 +46,8 @@ __host__ __device__ constexpr int swz(int row, int c) {
 
 // Cooperative direct global->LDS copy of a [ROWS x COLS] fp16 tile (row stride `ld` elements
 // in global memory) into a swizzled LDS tile with COLS-element rows.
-template <int ROWS, int COLS>
-TFK_DEVICE void tile_to_lds(const half_t* __restrict__ g, size_t ld, char* lds, int wave, int lane) {
+template <typename T, int ROWS, int COLS>
+TFK_DEVICE void tile_to_lds(const T* __restrict__ g, size_t ld, char* lds, int wave, int lane) {
   constexpr int CH = COLS / 8;
   constexpr int kRowsPerInstr = 64 / CH;
   constexpr int kInstr = ROWS * CH / 64;
@@ -56,15 +67,15 @@ TFK_DEVICE void tile_to_lds(const half_t* __restrict__ g, size_t ld, char* lds, 
 //   second_product: acc2[pt] += (fp16 of acc1) * C over the TN / 32 steps; lane (m = lr, group
 //                   lg) holds A*B[m][16*nt + 4*lg + r] in acc1[nt][r], and reduction step s uses
 //                   n = 32*s + {4*lg + 0..3, 16 + 4*lg + 0..3} as its 8 slots.
-template <int TN, int KC>
-TFK_DEVICE void first_product(const char* sB, const half8_t* af, float4_t* acc1, int lr, int lg) {
+template <typename T, int TN, int KC>
+TFK_DEVICE void first_product(const char* sB, const vec8_t<T>* af, float4_t* acc1, int lr, int lg) {
   constexpr int kNT = TN / 16, kKSteps = KC / 32, kCh = KC / 8;
-  half8_t bf[2][kNT];
+  vec8_t<T> bf[2][kNT];
   auto read_b = [&](int buf, int ks) __attribute__((always_inline)) {
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt) {
       const int row = nt * 16 + lr;
-      bf[buf][nt] = *reinterpret_cast<const half8_t*>(sB + row * KC * 2 + swz<kCh>(row, ks * 4 + lg) * 16);
+      bf[buf][nt] = *reinterpret_cast<const vec8_t<T>*>(sB + row * KC * 2 + swz<kCh>(row, ks * 4 + lg) * 16);
     }
   };
   read_b(0, 0);
@@ -72,21 +83,21 @@ TFK_DEVICE void first_product(const char* sB, const half8_t* af, float4_t* acc1,
   for (int ks = 0; ks < kKSteps; ++ks) {
     if (ks + 1 < kKSteps) read_b((ks + 1) & 1, ks + 1);
 #pragma unroll
-    for (int nt = 0; nt < kNT; ++nt) acc1[nt] = mfma_16x16x32(bf[ks & 1][nt], af[ks], acc1[nt]);
+    for (int nt = 0; nt < kNT; ++nt) acc1[nt] = mfma_t<T>(bf[ks & 1][nt], af[ks], acc1[nt]);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
-template <int TN, int TP>
+template <typename T, int TN, int TP>
 TFK_DEVICE void second_product(const char* sC, const float4_t* acc1, float4_t* acc2, int lr, int lg) {
   constexpr int kPT = TP / 16, kSteps = TN / 32, kCh = TN / 8;
-  half8_t cf[2][kPT];
+  vec8_t<T> cf[2][kPT];
   auto read_c = [&](int buf, int s2) __attribute__((always_inline)) {
 #pragma unroll
     for (int pt = 0; pt < kPT; ++pt) {
       const int row = pt * 16 + lr;
       const char* base = sC + row * TN * 2 + (lg & 1) * 8;
-      const half4_t lo = *reinterpret_cast<const half4_t*>(base + swz<kCh>(row, 4 * s2 + (lg >> 1)) * 16);
-      const half4_t hi = *reinterpret_cast<const half4_t*>(base + swz<kCh>(row, 4 * s2 + 2 + (lg >> 1)) * 16);
+      const vec4_t<T> lo = *reinterpret_cast<const vec4_t<T>*>(base + swz<kCh>(row, 4 * s2 + (lg >> 1)) * 16);
+      const vec4_t<T> hi = *reinterpret_cast<const vec4_t<T>*>(base + swz<kCh>(row, 4 * s2 + 2 + (lg >> 1)) * 16);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         cf[buf][pt][r] = lo[r];
@@ -98,14 +109,14 @@ TFK_DEVICE void second_product(const char* sC, const float4_t* acc1, float4_t* a
 #pragma unroll
   for (int s2 = 0; s2 < kSteps; ++s2) {
     if (s2 + 1 < kSteps) read_c((s2 + 1) & 1, s2 + 1);
-    half8_t pa;
+    vec8_t<T> pa;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      pa[r] = (half_t)acc1[2 * s2][r];
-      pa[4 + r] = (half_t)acc1[2 * s2 + 1][r];
+      pa[r] = (T)acc1[2 * s2][r];
+      pa[4 + r] = (T)acc1[2 * s2 + 1][r];
     }
 #pragma unroll
-    for (int pt = 0; pt < kPT; ++pt) acc2[pt] = mfma_16x16x32(pa, cf[s2 & 1][pt], acc2[pt]);
+    for (int pt = 0; pt < kPT; ++pt) acc2[pt] = mfma_t<T>(pa, cf[s2 & 1][pt], acc2[pt]);
     __builtin_amdgcn_sched_barrier(0);
   }
 }
@@ -138,10 +149,10 @@ __host__ __device__ constexpr int b_key(int row) {
   else return (row / (16 / CH)) % CH;
 }
 
-template <int TN, int TP, int KC>
+template <typename T, int TN, int TP, int KC>
 __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
-    const half_t* __restrict__ A, const half_t* __restrict__ B, const half_t* __restrict__ C,
-    half_t* __restrict__ D, int M, int N, int K, int P) {
+    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ C,
+    T* __restrict__ D, int M, int N, int K, int P) {
   constexpr int kBCh = KC / 8;       // 16-byte chunks per sB row
   constexpr int kCCh = TN / 8;       // per sC row
   constexpr int kKSteps = KC / 32;
@@ -208,18 +219,18 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
   // requests of this wavefront that are still allowed in flight when B (and A) must be there
   const int c_requests = (kCInstr % kWaves == 0 || wave < kCInstr % kWaves) ? kCPerWave : kCPerWave - 1;
 
-  auto read_b = [&](half8_t* dst, int ks) __attribute__((always_inline)) {
+  auto read_b = [&](vec8_t<T>* dst, int ks) __attribute__((always_inline)) {
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt) {
       const int row = b_frag_row(nt, lr);
-      dst[nt] = *reinterpret_cast<const half8_t*>(sB + row * KC * 2 + ((ks * 4 + lg) ^ b_key<kBCh>(row)) * 16);
+      dst[nt] = *reinterpret_cast<const vec8_t<T>*>(sB + row * KC * 2 + ((ks * 4 + lg) ^ b_key<kBCh>(row)) * 16);
     }
   };
-  auto read_c = [&](half8_t* dst, int s2) __attribute__((always_inline)) {
+  auto read_c = [&](vec8_t<T>* dst, int s2) __attribute__((always_inline)) {
 #pragma unroll
     for (int pt = 0; pt < kPT; ++pt) {
       const int row = pt * 16 + lr;
-      dst[pt] = *reinterpret_cast<const half8_t*>(sC + row * TN * 2 + swz<kCCh>(row, 4 * s2 + lg) * 16);
+      dst[pt] = *reinterpret_cast<const vec8_t<T>*>(sC + row * TN * 2 + swz<kCCh>(row, 4 * s2 + lg) * 16);
     }
   };
 
@@ -236,7 +247,7 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
       const bool first_chunk = k0 == 0;
       // previous readers of sB (and, at a new n-tile, of sC) are done
       if (n0 != 0 || k0 != 0) barrier_lds_only();
-      half8_t af[kKSteps];
+      vec8_t<T> af[kKSteps];
       // All three kinds of request are issued from assembly, so that the compiler places no
       // vector-memory waits of its own (it would drain everything, the C tile included, in
       // front of the first LDS read or the first use of an A fragment).
@@ -269,13 +280,13 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
       asm volatile("" ::: "memory");
 
       // first product, transposed: acc1[nt] += B rows (fragment nt) x A^T, reads one step ahead
-      half8_t bf[2][kNT];
+      vec8_t<T> bf[2][kNT];
       read_b(bf[0], 0);
 #pragma unroll
       for (int ks = 0; ks < kKSteps; ++ks) {
         if (ks + 1 < kKSteps) read_b(bf[(ks + 1) & 1], ks + 1);
 #pragma unroll
-        for (int nt = 0; nt < kNT; ++nt) acc1[nt] = mfma_16x16x32(bf[ks & 1][nt], af[ks], acc1[nt]);
+        for (int nt = 0; nt < kNT; ++nt) acc1[nt] = mfma_t<T>(bf[ks & 1][nt], af[ks], acc1[nt]);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -285,19 +296,19 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
     asm volatile("" ::: "memory");
     // second product, transposed: lane (m = lr, group lg) holds A*B[m][32*s2 + 8*lg + 0..7] in
     // acc1[2*s2][0..3], acc1[2*s2 + 1][0..3]; acc2[pt] += C rows (p) x that
-    half8_t cf[2][kPT];
+    vec8_t<T> cf[2][kPT];
     read_c(cf[0], 0);
 #pragma unroll
     for (int s2 = 0; s2 < kSteps2; ++s2) {
       if (s2 + 1 < kSteps2) read_c(cf[(s2 + 1) & 1], s2 + 1);
-      half8_t pa;
+      vec8_t<T> pa;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        pa[r] = (half_t)acc1[2 * s2][r];
-        pa[4 + r] = (half_t)acc1[2 * s2 + 1][r];
+        pa[r] = (T)acc1[2 * s2][r];
+        pa[4 + r] = (T)acc1[2 * s2 + 1][r];
       }
 #pragma unroll
-      for (int pt = 0; pt < kPT; ++pt) acc2[pt] = mfma_16x16x32(cf[s2 & 1][pt], pa, acc2[pt]);
+      for (int pt = 0; pt < kPT; ++pt) acc2[pt] = mfma_t<T>(cf[s2 & 1][pt], pa, acc2[pt]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -311,17 +322,17 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
     // that a store writes 16 rows x 64 contiguous bytes with four adjacent lanes per row.
     const int st_row = lane >> 2, st_seg = lane & 3;
     const int src_lane = st_row + 16 * (((st_seg & 1) << 1) | (st_seg >> 1));
-    half_t* d_lane = D + (size_t)(d_row0 + st_row) * P + p0 + 8 * st_seg;
+    T* d_lane = D + (size_t)(d_row0 + st_row) * P + p0 + 8 * st_seg;
     const bool row_ok = d_row0 + st_row < M;
     uint4_t v[kPT / 2];
 #pragma unroll
     for (int pt = 0; pt < kPT; pt += 2) {
-      typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+      typedef vec2_t<T> h2_t;
       unsigned x[2], y[2];
 #pragma unroll
       for (int d = 0; d < 2; ++d) {
-        const h2_t hx = {(half_t)acc2[pt][2 * d], (half_t)acc2[pt][2 * d + 1]};
-        const h2_t hy = {(half_t)acc2[pt + 1][2 * d], (half_t)acc2[pt + 1][2 * d + 1]};
+        const h2_t hx = {(T)acc2[pt][2 * d], (T)acc2[pt][2 * d + 1]};
+        const h2_t hy = {(T)acc2[pt + 1][2 * d], (T)acc2[pt + 1][2 * d + 1]};
         x[d] = __builtin_bit_cast(unsigned, hx);
         y[d] = __builtin_bit_cast(unsigned, hy);
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -346,22 +357,22 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
     // a single 16-column tile: 8 bytes per lane
 #pragma unroll
     for (int pt = 0; pt < kPT; ++pt) {
-      half4_t v;
+      vec4_t<T> v;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] = (half_t)acc2[pt][r];
+      for (int r = 0; r < 4; ++r) v[r] = (T)acc2[pt][r];
       if (d_row0 + lr < M)
-        *reinterpret_cast<half4_t*>(D + (size_t)(d_row0 + lr) * P + p0 + 16 * pt + 4 * lg) = v;
+        *reinterpret_cast<vec4_t<T>*>(D + (size_t)(d_row0 + lr) * P + p0 + 16 * pt + 4 * lg) = v;
     }
   }
 }
 
-template <int TN, int TP, int KC>
+template <typename T, int TN, int TP, int KC>
 int launch(const void* A, const void* B, const void* C, void* D, int batch, int M, int N, int K,
            int P, hipStream_t st) {
   dim3 grid((M + kRowsPerBlock - 1) / kRowsPerBlock, P / TP, batch);
-  hipLaunchKernelGGL((fused_two_gemms_kernel<TN, TP, KC>), grid, dim3(kThreads), 0, st,
-                     static_cast<const half_t*>(A), static_cast<const half_t*>(B),
-                     static_cast<const half_t*>(C), static_cast<half_t*>(D), M, N, K, P);
+  hipLaunchKernelGGL((fused_two_gemms_kernel<T, TN, TP, KC>), grid, dim3(kThreads), 0, st,
+                     static_cast<const T*>(A), static_cast<const T*>(B),
+                     static_cast<const T*>(C), static_cast<T*>(D), M, N, K, P);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
 }
@@ -382,10 +393,10 @@ int launch(const void* A, const void* B, const void* C, void* D, int batch, int 
 // partial sums to part blockIdx.y of the workspace W [batch][parts][M][128] instead of D; a second
 // kernel adds the parts up.  M / 64 workgroups do not fill the chip for the shapes this kernel is
 // for, and a workgroup is bound by how many tile bytes its ring keeps in flight, not by arithmetic.
-template <int kWavesT, int kSplit, bool kPartial>
+template <typename T, int kWavesT, int kSplit, bool kPartial>
 __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_kernel(
-    const half_t* __restrict__ A, const half_t* __restrict__ B, const half_t* __restrict__ C,
-    half_t* __restrict__ D, float* __restrict__ W, int M, int N, int tiles_per_part) {
+    const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ C,
+    T* __restrict__ D, float* __restrict__ W, int M, int N, int tiles_per_part) {
   constexpr int K = 128, P = 128, TN = 64, kStagesS = 4;
   constexpr int kRows = 16 * kWavesT;
   constexpr int kBBytes = TN * K * 2;                // 16 KiB: B tile [n][k], 256-byte rows
@@ -401,7 +412,7 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
   // vmcnt allows 63 requests of one wavefront to stay in flight behind the awaited tile
   constexpr int kAhead = (kStagesS - 2) * kReqPerWave <= 63 ? kStagesS - 1 : 63 / kReqPerWave + 1;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  half_t* sD = reinterpret_cast<half_t*>(smem + kStagesS * kStageBytes);
+  T* sD = reinterpret_cast<T*>(smem + kStagesS * kStageBytes);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave = wave_id % kWavesT;      // which 16 rows
@@ -416,10 +427,10 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
   const unsigned smem_base = lds_address(smem);
 
   const int a_row = min(m0 + wave * 16 + lr, M - 1);  // clamped: rows past M are never stored
-  half8_t af[4];
+  vec8_t<T> af[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks)
-    af[ks] = *reinterpret_cast<const half8_t*>(A + (size_t)a_row * K + 8 * lg + ks * 32);
+    af[ks] = *reinterpret_cast<const vec8_t<T>*>(A + (size_t)a_row * K + 8 * lg + ks * 32);
 
   // this workgroup's n-tiles: [t_begin, t_begin + n_tiles)
   const int t_begin = kPartial ? (int)blockIdx.y * tiles_per_part : 0;
@@ -483,8 +494,8 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
     float4_t acc1[TN / 16];
 #pragma unroll
     for (int nt = 0; nt < TN / 16; ++nt) acc1[nt] = float4_t{0.f, 0.f, 0.f, 0.f};
-    first_product<TN, K>(sB, af, acc1, lr, lg);
-    second_product<TN, P>(sC, acc1, acc2, lr, lg);
+    first_product<T, TN, K>(sB, af, acc1, lr, lg);
+    second_product<T, TN, P>(sC, acc1, acc2, lr, lg);
   }
   wait_vmem_all();  // the surplus requests must not outlive the workgroup's LDS
   if constexpr (kSplit > 1) {
@@ -525,7 +536,7 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
 #pragma unroll
     for (int pt = 0; pt < 8; ++pt)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sD[(wave * 16 + 4 * lg + r) * P + pt * 16 + lr] = (half_t)acc2[pt][r];
+      for (int r = 0; r < 4; ++r) sD[(wave * 16 + 4 * lg + r) * P + pt * 16 + lr] = (T)acc2[pt][r];
   }
   __syncthreads();
   constexpr int kDChunks = P / 8;
@@ -538,8 +549,9 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
 }
 
 // D[b][i] = fp16(sum over parts of W[b][part][i]), i over the M * 128 elements of a problem
+template <typename T>
 __global__ __launch_bounds__(256) void fused_two_gemms_reduce_kernel(const float* __restrict__ W,
-                                                                     half_t* __restrict__ D, int parts,
+                                                                     T* __restrict__ D, int parts,
                                                                      size_t elems) {
   const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= elems) return;
@@ -547,21 +559,21 @@ __global__ __launch_bounds__(256) void fused_two_gemms_reduce_kernel(const float
   float4_t acc = __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(w));
   for (int part = 1; part < parts; ++part)
     acc += __builtin_nontemporal_load(reinterpret_cast<const float4_t*>(w + (size_t)part * elems));
-  half4_t h = {(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
-  *reinterpret_cast<half4_t*>(D + (size_t)blockIdx.z * elems + i) = h;
+  vec4_t<T> h = {(T)acc[0], (T)acc[1], (T)acc[2], (T)acc[3]};
+  *reinterpret_cast<vec4_t<T>*>(D + (size_t)blockIdx.z * elems + i) = h;
 }
 
-template <int kWavesT, int kSplit>
+template <typename T, int kWavesT, int kSplit>
 int launch_stream(const void* A, const void* B, const void* C, void* D, int batch, int M, int N,
                   hipStream_t st) {
-  auto kern = fused_two_gemms_stream_kernel<kWavesT, kSplit, false>;
+  auto kern = fused_two_gemms_stream_kernel<T, kWavesT, kSplit, false>;
   constexpr int lds = 4 * (64 * 128 * 2 + 128 * 64 * 2) + 16 * kWavesT * 128 * 2;
   static_assert(lds <= kMaxLdsBytes, "ring does not fit in LDS");
   TFK_LDS_OPT_IN(kern, lds);
   dim3 grid((M + 16 * kWavesT - 1) / (16 * kWavesT), 1, batch);
-  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const half_t*>(A),
-                     static_cast<const half_t*>(B), static_cast<const half_t*>(C),
-                     static_cast<half_t*>(D), static_cast<float*>(nullptr), M, N, 0);
+  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const T*>(A),
+                     static_cast<const T*>(B), static_cast<const T*>(C),
+                     static_cast<T*>(D), static_cast<float*>(nullptr), M, N, 0);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
 }
@@ -599,37 +611,37 @@ SplitPlan fused_split_plan(int64_t batch, int64_t M, int64_t N, int64_t K, int64
   return plan;
 }
 
-template <int kWavesT, int kSplit>
+template <typename T, int kWavesT, int kSplit>
 int launch_stream_split(const void* A, const void* B, const void* C, void* D, float* W, SplitPlan plan, int batch,
                         int M, int N, hipStream_t st) {
-  auto kern = fused_two_gemms_stream_kernel<kWavesT, kSplit, true>;
+  auto kern = fused_two_gemms_stream_kernel<T, kWavesT, kSplit, true>;
   constexpr int lds = 4 * (64 * 128 * 2 + 128 * 64 * 2) + 16 * kWavesT * 128 * 2;
   TFK_LDS_OPT_IN(kern, lds);
   dim3 grid((M + 16 * kWavesT - 1) / (16 * kWavesT), plan.parts, batch);
-  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const half_t*>(A),
-                     static_cast<const half_t*>(B), static_cast<const half_t*>(C),
-                     static_cast<half_t*>(D), W, M, N, plan.tiles_per_part);
+  hipLaunchKernelGGL(kern, grid, dim3(kWavesT * kSplit * 64), lds, st, static_cast<const T*>(A),
+                     static_cast<const T*>(B), static_cast<const T*>(C),
+                     static_cast<T*>(D), W, M, N, plan.tiles_per_part);
   TFK_HIP_TRY(hipGetLastError());
   const size_t elems = (size_t)M * 128;
-  hipLaunchKernelGGL(fused_two_gemms_reduce_kernel, dim3((unsigned)((elems / 4 + 255) / 256), 1, batch), dim3(256), 0,
-                     st, W, static_cast<half_t*>(D), plan.parts, elems);
+  hipLaunchKernelGGL(fused_two_gemms_reduce_kernel<T>, dim3((unsigned)((elems / 4 + 255) / 256), 1, batch), dim3(256), 0,
+                     st, W, static_cast<T*>(D), plan.parts, elems);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
 }
 
-template <int TN, int TP>
+template <typename T, int TN, int TP>
 int pick_kc(const void* A, const void* B, const void* C, void* D, int batch, int M, int N, int K,
             int P, hipStream_t st) {
-  if (K % 128 == 0) return launch<TN, TP, 128>(A, B, C, D, batch, M, N, K, P, st);
-  return launch<TN, TP, 32>(A, B, C, D, batch, M, N, K, P, st);
+  if (K % 128 == 0) return launch<T, TN, TP, 128>(A, B, C, D, batch, M, N, K, P, st);
+  return launch<T, TN, TP, 32>(A, B, C, D, batch, M, N, K, P, st);
 }
 
-template <int TN>
+template <typename T, int TN>
 int pick_tp(const void* A, const void* B, const void* C, void* D, int batch, int M, int N, int K,
             int P, hipStream_t st) {
-  if (P % 128 == 0) return pick_kc<TN, 128>(A, B, C, D, batch, M, N, K, P, st);
-  if (P % 64 == 0) return pick_kc<TN, 64>(A, B, C, D, batch, M, N, K, P, st);
-  return pick_kc<TN, 16>(A, B, C, D, batch, M, N, K, P, st);
+  if (P % 128 == 0) return pick_kc<T, TN, 128>(A, B, C, D, batch, M, N, K, P, st);
+  if (P % 64 == 0) return pick_kc<T, TN, 64>(A, B, C, D, batch, M, N, K, P, st);
+  return pick_kc<T, TN, 16>(A, B, C, D, batch, M, N, K, P, st);
 }
 
 }  // namespace
@@ -655,29 +667,45 @@ int check_fused_args(const char* who, const void* A, const void* B, const void* 
 }  // namespace
 }  // namespace tfk
 
-extern "C" int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, void* D,
-                                      int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P,
-                                      int tm, int tn, int tk, int tp, void* stream) {
-  using namespace tfk;
-  if (int rc = check_fused_args("tf_fused_two_gemms_f16", A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp)) return rc;
-  hipStream_t st = static_cast<hipStream_t>(stream);
+namespace tfk {
+namespace {
+// the tuned kernels for element type T (arguments already checked)
+template <typename T>
+int run_fused(const void* A, const void* B, const void* C, void* D, int64_t batch, int64_t M, int64_t N, int64_t K,
+              int64_t P, hipStream_t st) {
   // long N: stream the B / C tiles through the LDS ring (8-15% faster than the plain kernel's
   // load - wait - multiply per n-tile; both are bound by the latencies of one wavefront per SIMD)
   if (K == 128 && P == 128 && N % 64 == 0 && N >= 256) {
     // enough rows for a 128-row block per CU: eight wavefronts share every tile (1.23 us per tile
     // for 128 rows against 0.8 us for 64)
     if (N >= 512 && (M + 127) / 128 * batch >= 256)
-      return launch_stream<8, 1>(A, B, C, D, (int)batch, (int)M, (int)N, st);
-    return launch_stream<4, 2>(A, B, C, D, (int)batch, (int)M, (int)N, st);
+      return launch_stream<T, 8, 1>(A, B, C, D, (int)batch, (int)M, (int)N, st);
+    return launch_stream<T, 4, 2>(A, B, C, D, (int)batch, (int)M, (int)N, st);
   }
-  if (N % 128 == 0) return pick_tp<128>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
-  return pick_tp<32>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
+  if (N % 128 == 0) return pick_tp<T, 128>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
+  return pick_tp<T, 32>(A, B, C, D, (int)batch, (int)M, (int)N, (int)K, (int)P, st);
+}
+template <typename T>
+int run_fused_split(const void* A, const void* B, const void* C, void* D, float* W, SplitPlan plan, int64_t batch,
+                    int64_t M, int64_t N, hipStream_t st) {
+  if (plan.rows == 128) return launch_stream_split<T, 8, 1>(A, B, C, D, W, plan, (int)batch, (int)M, (int)N, st);
+  return launch_stream_split<T, 4, 2>(A, B, C, D, W, plan, (int)batch, (int)M, (int)N, st);
+}
+}  // namespace
+}  // namespace tfk
+
+extern "C" int tf_fused_two_gemms_f16(const void* A, const void* B, const void* C, void* D,
+                                      int64_t batch, int64_t M, int64_t N, int64_t K, int64_t P,
+                                      int tm, int tn, int tk, int tp, void* stream) {
+  using namespace tfk;
+  if (int rc = check_fused_args("tf_fused_two_gemms_f16", A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp)) return rc;
+  return run_fused<half_t>(A, B, C, D, batch, M, N, K, P, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t tf_fused_two_gemms_workspace_bytes(int dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
                                                      int64_t P) {
   using namespace tfk;
-  if (dtype != TF_DTYPE_F16 || batch <= 0 || M <= 0 || N <= 0) return 0;
+  if ((dtype != TF_DTYPE_F16 && dtype != TF_DTYPE_BF16) || batch <= 0 || M <= 0 || N <= 0) return 0;
   const SplitPlan plan = fused_split_plan(batch, M, N, K, P);
   return plan.parts > 1 ? (size_t)plan.parts * (size_t)batch * (size_t)M * 128 * sizeof(float) : 0;
 }
@@ -693,11 +721,10 @@ extern "C" int tf_fused_two_gemms_ws(const void* A, const void* B, const void* C
   TFK_REQUIRE(reinterpret_cast<uintptr_t>(workspace) % 16 == 0, TF_ERR_INVALID_ARG,
               "tf_fused_two_gemms_ws: workspace must be 16-byte aligned");
   const SplitPlan plan = fused_split_plan(batch, M, N, K, P);
-  if (plan.rows == 128)
-    return launch_stream_split<8, 1>(A, B, C, D, static_cast<float*>(workspace), plan, (int)batch, (int)M, (int)N,
-                                     static_cast<hipStream_t>(stream));
-  return launch_stream_split<4, 2>(A, B, C, D, static_cast<float*>(workspace), plan,
-                                   (int)batch, (int)M, (int)N, static_cast<hipStream_t>(stream));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == TF_DTYPE_BF16)
+    return run_fused_split<bf16_t>(A, B, C, D, static_cast<float*>(workspace), plan, batch, M, N, st);
+  return run_fused_split<half_t>(A, B, C, D, static_cast<float*>(workspace), plan, batch, M, N, st);
 }
 
 extern "C" int tf_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype, int64_t batch,
@@ -707,7 +734,7 @@ extern "C" int tf_fused_two_gemms(const void* A, const void* B, const void* C, v
   if (dtype == TF_DTYPE_F16) return tf_fused_two_gemms_f16(A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp, stream);
   TFK_REQUIRE(dtype == TF_DTYPE_BF16, TF_ERR_UNSUPPORTED,
               "tf_fused_two_gemms: dtype must be TF_DTYPE_F16 or TF_DTYPE_BF16");
+  // bf16: the same kernels with the bf16 MFMA, a bf16 intermediate and bf16 output
   if (int rc = check_fused_args("tf_fused_two_gemms", A, B, C, D, batch, M, N, K, P, tm, tn, tk, tp)) return rc;
-  TFK_REQUIRE(jit_fused_supports(M, N, K, P), TF_ERR_UNSUPPORTED, "tf_fused_two_gemms: bf16 needs M %% 16 == 0");
-  return jit_fused_two_gemms(A, B, C, D, dtype, batch, M, N, K, P, tm, tn, tk, tp, static_cast<hipStream_t>(stream));
+  return run_fused<bf16_t>(A, B, C, D, batch, M, N, K, P, static_cast<hipStream_t>(stream));
 }

@@ -137,34 +137,4 @@ int jit_gemm(const void* A, const void* B, void* C, int dtype, int c_kind, int64
                             st);
 }
 
-bool jit_fused_supports(int64_t M, int64_t N, int64_t K, int64_t P) {
-  return M % 16 == 0 && N % 32 == 0 && K % 32 == 0 && P % 16 == 0;
-}
-
-int jit_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype, int64_t batch, int64_t M,
-                        int64_t N, int64_t K, int64_t P, int tm, int tn, int tk, int tp, hipStream_t st) {
-  if (tm % 16 != 0 || M % tm != 0 || tm > 128) tm = pick_divisor(M, {64, 32, 16});
-  if (tn % 32 != 0 || N % tn != 0 || tn > 128) tn = pick_divisor(N, {64, 32});
-  if (tk % 32 != 0 || K % tk != 0 || tk > 128) tk = pick_divisor(K, {64, 32});
-  if (tp % 16 != 0 || P % tp != 0 || tp > 128) tp = pick_divisor(P, {64, 32, 16});
-  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0 && tp > 0, TF_ERR_UNSUPPORTED,
-              "fused_two_gemms: no legal tiling for M=%lld N=%lld K=%lld P=%lld", (long long)M, (long long)N,
-              (long long)K, (long long)P);
-  int wr = tm / 16 > 4 ? 4 : tm / 16;
-  while ((tm / wr) % 16 != 0) --wr;
-  const char* T = type_name(dtype);
-  std::ostringstream name, src;
-  name << "tf_fused_" << (dtype == TF_DTYPE_BF16 ? "bf16_" : "f16_") << M << "_" << N << "_" << K << "_" << P << "_" << tm
-       << "_" << tn << "_" << tk << "_" << tp << "_" << wr;
-  src << kPrelude << "using Config = FusedTwoGemmsTraits<" << T << ", float, tl::RowMajor<" << wr << ", 1>, " << M << ", "
-      << N << ", " << K << ", " << P << ", " << tm << ", " << tn << ", " << tk << ", " << tp << ">;\n"
-      << "extern \"C\" __global__ __launch_bounds__(" << wr * 64 << ") void " << name.str() << "(const " << T
-      << "* A, const " << T << "* B, const " << T << "* C, " << T << "* D) {\n"
-      << "  ke_fused_two_gemms<" << T << ", float, Config>(A, B, C, D);\n}\n";
-  const unsigned lds = (unsigned)(tm * tk + tk * tn + tn * tp + tm * tn) * 2u;
-  void* args[] = {&A, &B, &C, &D};
-  return compile_and_launch(name.str(), src.str(), dim3((unsigned)(M / tm), (unsigned)(P / tp), (unsigned)batch),
-                            wr * 64, lds, args, st);
-}
-
 }  // namespace tfk

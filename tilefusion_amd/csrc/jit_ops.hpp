@@ -13,10 +13,6 @@ bool jit_gemm_supports(int64_t M, int64_t N, int64_t K);
 int jit_gemm(const void* A, const void* B, void* C, int dtype, int c_kind, int64_t M, int64_t N, int64_t K, int tm,
              int tn, int tk, int num_stages, int pipeline_level, hipStream_t st);
 
-bool jit_fused_supports(int64_t M, int64_t N, int64_t K, int64_t P);
-int jit_fused_two_gemms(const void* A, const void* B, const void* C, void* D, int dtype, int64_t batch, int64_t M,
-                        int64_t N, int64_t K, int64_t P, int tm, int tn, int tk, int tp, hipStream_t st);
-
 // V must be handed over transposed ([batch, Dv, Lkv])
 bool jit_flash_attention_supports(int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int v_is_transposed);
 int jit_flash_attention(const void* Q, const void* K, const void* Vt, void* O, int dtype, int64_t batch, int64_t Lq,

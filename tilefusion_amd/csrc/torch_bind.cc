@@ -118,10 +118,10 @@ void fused_two_gemms(const at::Tensor& A, const at::Tensor& B, const at::Tensor&
               "batch dimensions must match.");
   // The kernels reduce 32 values of k (and of n, in the second product) per MFMA and write 16
   // columns per base tile.  Shapes the reference accepts with 16-wide base tiles (K or N = 48,
-  // ...) are zero-padded here: zeros add nothing to either product.  A padded P or M (bf16:
-  // 16 rows per wavefront) goes through a temporary D.
+  // ...) are zero-padded here: zeros add nothing to either product.  A padded P goes through a
+  // temporary D.
   const int64_t kp = round_up(k, 32), np = round_up(n, 32), pp = round_up(p, 16);
-  const int64_t mp = dtype == TF_DTYPE_BF16 ? round_up(m, 16) : m;
+  const int64_t mp = m;
   if (kp == k && np == n && pp == p && mp == m) {
     // long-N problems are cut along N when the library is handed a workspace for the partial sums
     const size_t ws_bytes = tf_fused_two_gemms_workspace_bytes(dtype, batch, m, n, k, p);
