@@ -97,7 +97,7 @@ class Gemm4096:
     bytes = 3 * 4096 * 4096 * 2
     # Measured bytes per launch between the L2 caches and the fabric (rocprofv3 FETCH_SIZE +
     # WRITE_SIZE, each scaled by what it reads for a 1 GiB copy; summaries under profiles/).
-    traffic = 235087391
+    traffic = 235087049
 
     def setup(self, dev):
         import torch
@@ -141,7 +141,7 @@ class Fused:
     M, N, K, P = 16384, 128, 128, 128
     flops = 2.0 * 2 * 16384 * 128 * 128
     bytes = (16384 * 128 * 2 + 2 * 128 * 128) * 2
-    traffic = 9372637  # measured, see Gemm4096.traffic
+    traffic = 9067224  # measured, see Gemm4096.traffic
 
     def setup(self, dev):
         import torch
@@ -185,7 +185,7 @@ class Attention:
         self.metric = "flash_attention_fwd_tflops" + ("_causal" if causal else "")
         self.flops = 4.0 * 64 * 4096 * 4096 * 128 * (0.5 if causal else 1.0)
         self.bytes = 4 * 64 * 4096 * 128 * 2
-        self.traffic = 384475716 if causal else 268696520  # measured, see Gemm4096.traffic
+        self.traffic = 384216579 if causal else 268700488  # measured, see Gemm4096.traffic
         self.config = {"workload": "flash-attention fwd fp16 B=2 H=32 S=4096 D=128 %s, scale 1/sqrt(128), fp32 softmax stats"
                        % ("causal" if causal else "non-causal"),
                        "inputs": "N(0,1), seed 1004; V in natural [S, D] layout; 2 rotating Q/K/V/O sets"}
@@ -240,7 +240,7 @@ class Decode:
     BH, LKV, D, SPLITS = 512, 32768, 128, 64
     bytes = 2 * 512 * 32768 * 128 * 2 + 2 * 512 * 128 * 2
     flops = 4.0 * 512 * 32768 * 128
-    traffic = 8626356157  # both kernels of a step; measured, see Gemm4096.traffic
+    traffic = 8626347552  # both kernels of a step; measured, see Gemm4096.traffic
 
     def setup(self, dev):
         import torch
