@@ -50,10 +50,7 @@ TF_API int tf_gemm_f16(const void* A, const void* B, void* C, int c_is_f16, int6
 /* The same for fp16 or bf16 inputs (dtype = TF_DTYPE_F16 / TF_DTYPE_BF16, the reference's declared
  * type set, include/kernels/dispatch_macros.hpp:6-23 and include/cell/compute/gemm.hpp:107-150):
  * C is fp32 when c_is_f32 != 0, else of the input type.  fp16 is tf_gemm_f16.  bf16 runs the same
- * ring kernel with v_mfma_f32_16x16x32_bf16 when M, N are multiples of 128 and K of 64; other
- * bf16 shapes (M, N multiples of 16, K of 32) are compiled at run time from the header kernel
- * with the caller's tile sizes (first call per shape: seconds, then cached in the process and on
- * disk). */
+ * kernels with the bf16 MFMAs (any M, N; K a multiple of 8). */
 TF_API int tf_gemm(const void* A, const void* B, void* C, int dtype, int c_is_f32, int64_t M,
                    int64_t N, int64_t K, int tm, int tn, int tk, int num_stages,
                    int pipeline_level, void* stream);

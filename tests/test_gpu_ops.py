@@ -167,9 +167,12 @@ def test_fused_two_gemms_op_pads_what_the_kernels_cannot_tile(m, n, k, p):
     assert ok, (r, mx)
 
 
-@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (4096, 512, 256), (96, 160, 64), (128, 128, 96)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 128), (4096, 512, 256), (96, 160, 64), (128, 128, 96),
+                                   (4096, 2048, 96), (32, 32, 32)])
 def test_gemm_op_bf16(m, n, k):
-    # the first two shapes run the ring kernel with the bf16 MFMA, the others the run-time compiled one
+    # every kernel of the GEMM is a template of the operand type: the ring kernel (first two shapes),
+    # the bounds-checked kernel (96 x 160), the 32-deep direct-to-LDS kernels with 128- and 256-wide
+    # tiles (K = 96)
     from tilefusion_amd.ops import gemm
     a, b = oracle.make_c1_gemm_inputs(m, n, k, seed=77)
     a, b = a.bfloat16(), b.bfloat16()

@@ -22,7 +22,6 @@
 #include <type_traits>
 
 #include "common.hpp"
-#include "jit_ops.hpp"
 
 namespace tfk {
 namespace {
@@ -79,6 +78,19 @@ TFK_DEVICE void store_out(OutT* p, float v) {
   }
 }
 
+// MFMAs by operand type (half_t or bf16_t) for the kernels that issue them through builtins
+template <typename InT> using in8_t = InT __attribute__((ext_vector_type(8)));
+template <typename InT>
+TFK_DEVICE float4_t mfma16_t(in8_t<InT> a, in8_t<InT> b, float4_t c) {
+  if constexpr (std::is_same_v<InT, bf16_t>) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  else return mfma_16x16x32(a, b, c);
+}
+template <typename InT>
+TFK_DEVICE float16_t mfma32_t(in8_t<InT> a, in8_t<InT> b, float16_t c) {
+  if constexpr (std::is_same_v<InT, bf16_t>) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  else return mfma_32x32x16(a, b, c);
+}
+
 // ------------------------------------------------------------------------------------------
 // Fast path: M % BM == 0, N % BN == 0, K % 32 == 0.  Direct global->LDS ring, 16x16x32 MFMA.
 // ------------------------------------------------------------------------------------------
@@ -125,9 +137,9 @@ struct DirectShape {
   }
 };
 
-template <typename S, typename OutT>
+template <typename S, typename OutT, typename InT>
 __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
-    const half_t* __restrict__ A, const half_t* __restrict__ B, OutT* __restrict__ C, int M,
+    const InT* __restrict__ A, const InT* __restrict__ B, OutT* __restrict__ C, int M,
     int N, int K, int tiles_m, int tiles_n) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int tid = threadIdx.x;
@@ -216,7 +228,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
   constexpr int kInFlightAtBarrier =
       NS >= 3 ? (NS - 3) * kLoadsPerTile + kBarrierSlot * kLoadsPerTile / kSlots : 0;
   const int num_k_tiles = K / S::BK;
-  half8_t af[2][S::TM], bf[2][S::TN];
+  in8_t<InT> af[2][S::TM], bf[2][S::TN];
 
   auto issue_load = [&](int stage, int k0, int n) __attribute__((always_inline)) {
     char* sa = smem + stage * S::kStageBytes;
@@ -240,8 +252,8 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
     constexpr int kPerSlot = (kTotal + S::TM - 1) / S::TM;
 #pragma unroll
     for (int f = i * kPerSlot; f < (i + 1) * kPerSlot && f < kTotal; ++f) {
-      if (f < S::TN) bf[buf][f] = *reinterpret_cast<const half8_t*>(sb + b_rd[ks] + f * 16 * S::BK * 2);
-      else af[buf][f - S::TN] = *reinterpret_cast<const half8_t*>(sa + a_rd[ks] + (f - S::TN) * 16 * S::BK * 2);
+      if (f < S::TN) bf[buf][f] = *reinterpret_cast<const in8_t<InT>*>(sb + b_rd[ks] + f * 16 * S::BK * 2);
+      else af[buf][f - S::TN] = *reinterpret_cast<const in8_t<InT>*>(sa + a_rd[ks] + (f - S::TN) * 16 * S::BK * 2);
     }
   };
   // Past the end the schedule keeps running on a clamped tile index: the extra loads land in
@@ -289,7 +301,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
       if (ks + 1 < KS) load_frags(stage, ks + 1, cur ^ 1, i);
       else load_frags(stage_next, 0, cur ^ 1, i);
 #pragma unroll
-      for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma_16x16x32(bf[cur][j], af[cur][i], acc[i][j]);
+      for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma16_t<InT>(bf[cur][j], af[cur][i], acc[i][j]);
     }
   };
   int kt = 0;
@@ -310,10 +322,11 @@ __global__ __launch_bounds__(S::kThreads) void gemm_direct_lds_kernel(
     for (int j = 0; j < S::TN; ++j) {
       OutT* dst = C + (size_t)(c_row0 + 16 * i) * N + c_col0 + 16 * j;
       if constexpr (sizeof(OutT) == 2) {
-        half4_t v;
+        typedef OutT out4_t __attribute__((ext_vector_type(4)));
+        out4_t v;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = (half_t)acc[i][j][r];
-        *reinterpret_cast<half4_t*>(dst) = v;
+        for (int r = 0; r < 4; ++r) v[r] = (OutT)acc[i][j][r];
+        *reinterpret_cast<out4_t*>(dst) = v;
       } else {
         *reinterpret_cast<float4_t*>(dst) = acc[i][j];
       }
@@ -716,9 +729,9 @@ int launch_ring64(const void* A, const void* B, void* C, int M, int N, int K, hi
 // ------------------------------------------------------------------------------------------
 // General path: any M, N; K % 8 == 0.  Register-staged, bounds-checked, one LDS stage.
 // ------------------------------------------------------------------------------------------
-template <typename S, typename OutT>
+template <typename S, typename OutT, typename InT>
 __global__ __launch_bounds__(S::kThreads) void gemm_guarded_kernel(
-    const half_t* __restrict__ A, const half_t* __restrict__ B, OutT* __restrict__ C, int M,
+    const InT* __restrict__ A, const InT* __restrict__ B, OutT* __restrict__ C, int M,
     int N, int K) {
   __shared__ __attribute__((aligned(16))) char sa[S::kABytes];
   __shared__ __attribute__((aligned(16))) char sb[S::kBBytes];
@@ -755,21 +768,21 @@ __global__ __launch_bounds__(S::kThreads) void gemm_guarded_kernel(
     __syncthreads();
 #pragma unroll
     for (int kk = 0; kk < S::kKSteps; ++kk) {
-      half8_t af[S::TM], bf[S::TN];
+      in8_t<InT> af[S::TM], bf[S::TN];
 #pragma unroll
       for (int i = 0; i < S::TM; ++i) {
         const int row = wm * S::WM + i * 32 + fr;
-        af[i] = *reinterpret_cast<const half8_t*>(sa + row * S::BK * 2 + S::swizzle(row, 2 * kk + fg) * 16);
+        af[i] = *reinterpret_cast<const in8_t<InT>*>(sa + row * S::BK * 2 + S::swizzle(row, 2 * kk + fg) * 16);
       }
 #pragma unroll
       for (int j = 0; j < S::TN; ++j) {
         const int row = wn * S::WN + j * 32 + fr;
-        bf[j] = *reinterpret_cast<const half8_t*>(sb + row * S::BK * 2 + S::swizzle(row, 2 * kk + fg) * 16);
+        bf[j] = *reinterpret_cast<const in8_t<InT>*>(sb + row * S::BK * 2 + S::swizzle(row, 2 * kk + fg) * 16);
       }
 #pragma unroll
       for (int i = 0; i < S::TM; ++i)
 #pragma unroll
-        for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma_32x32x16(af[i], bf[j], acc[i][j]);
+        for (int j = 0; j < S::TN; ++j) acc[i][j] = mfma32_t<InT>(af[i], bf[j], acc[i][j]);
     }
     __syncthreads();
   }
@@ -790,25 +803,25 @@ using ShapeBig = DirectShape<256, 256, 32, 2, 2, 4>;         // 4 x 32 KiB of LD
 using ShapeMid = DirectShape<128, 128, 32, 2, 2, 4>;      // 4 x 16 KiB, 64x64 per wavefront
 using ShapeSmall = GemmShape<64, 64, 32, 2, 2, 1>;    // bounds-checked path
 
-template <typename S, typename OutT>
+template <typename S, typename OutT, typename InT>
 int launch_direct(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
-  auto kern = gemm_direct_lds_kernel<S, OutT>;
+  auto kern = gemm_direct_lds_kernel<S, OutT, InT>;
   constexpr int lds = S::kStages * S::kStageBytes;
   static_assert(lds <= kMaxLdsBytes, "tile does not fit in LDS");
   TFK_LDS_OPT_IN(kern, lds);
   const int tiles_m = M / S::BM, tiles_n = N / S::BN;
   hipLaunchKernelGGL(kern, dim3(tiles_m * tiles_n), dim3(S::kThreads), lds, st,
-                     static_cast<const half_t*>(A), static_cast<const half_t*>(B),
+                     static_cast<const InT*>(A), static_cast<const InT*>(B),
                      static_cast<OutT*>(C), M, N, K, tiles_m, tiles_n);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
 }
 
-template <typename S, typename OutT>
+template <typename S, typename OutT, typename InT>
 int launch_guarded(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
   dim3 grid((M + S::BM - 1) / S::BM, (N + S::BN - 1) / S::BN);
-  hipLaunchKernelGGL((gemm_guarded_kernel<S, OutT>), grid, dim3(S::kThreads), 0, st,
-                     static_cast<const half_t*>(A), static_cast<const half_t*>(B),
+  hipLaunchKernelGGL((gemm_guarded_kernel<S, OutT, InT>), grid, dim3(S::kThreads), 0, st,
+                     static_cast<const InT*>(A), static_cast<const InT*>(B),
                      static_cast<OutT*>(C), M, N, K);
   TFK_HIP_TRY(hipGetLastError());
   return TF_OK;
@@ -833,14 +846,14 @@ int dispatch_ring64(const void* A, const void* B, void* C, int M, int N, int K, 
   return launch_ring64<RingMid, OutT, InT>(A, B, C, M, N, K, st);
 }
 
-template <typename OutT>
+template <typename OutT, typename InT>
 int dispatch(const void* A, const void* B, void* C, int M, int N, int K, hipStream_t st) {
-  if (ring64_fits(M, N, K)) return dispatch_ring64<OutT, half_t>(A, B, C, M, N, K, st);
+  if (ring64_fits(M, N, K)) return dispatch_ring64<OutT, InT>(A, B, C, M, N, K, st);
   if (M % 256 == 0 && N % 256 == 0 && K % ShapeBig::BK == 0 && (int64_t)(M / 256) * (N / 256) >= 128)
-    return launch_direct<ShapeBig, OutT>(A, B, C, M, N, K, st);
+    return launch_direct<ShapeBig, OutT, InT>(A, B, C, M, N, K, st);
   if (M % 128 == 0 && N % 128 == 0 && K % 32 == 0)
-    return launch_direct<ShapeMid, OutT>(A, B, C, M, N, K, st);
-  return launch_guarded<ShapeSmall, OutT>(A, B, C, M, N, K, st);
+    return launch_direct<ShapeMid, OutT, InT>(A, B, C, M, N, K, st);
+  return launch_guarded<ShapeSmall, OutT, InT>(A, B, C, M, N, K, st);
 }
 
 }  // namespace
@@ -873,8 +886,8 @@ extern "C" int tf_gemm_f16(const void* A, const void* B, void* C, int c_is_f16, 
   TFK_REQUIRE(K % 8 == 0, TF_ERR_UNSUPPORTED, "tf_gemm_f16: K (%lld) must be a multiple of 8",
               (long long)K);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (c_is_f16) return dispatch<half_t>(A, B, C, (int)M, (int)N, (int)K, st);
-  return dispatch<float>(A, B, C, (int)M, (int)N, (int)K, st);
+  if (c_is_f16) return dispatch<half_t, half_t>(A, B, C, (int)M, (int)N, (int)K, st);
+  return dispatch<float, half_t>(A, B, C, (int)M, (int)N, (int)K, st);
 }
 
 extern "C" int tf_gemm(const void* A, const void* B, void* C, int dtype, int c_is_f32, int64_t M, int64_t N,
@@ -885,14 +898,9 @@ extern "C" int tf_gemm(const void* A, const void* B, void* C, int dtype, int c_i
   TFK_REQUIRE(dtype == TF_DTYPE_BF16, TF_ERR_UNSUPPORTED, "tf_gemm: dtype must be TF_DTYPE_F16 or TF_DTYPE_BF16");
   if (int rc = check_gemm_args("tf_gemm", A, B, C, M, N, K, tm, tn, tk, num_stages, pipeline_level)) return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  // bf16: the ring kernel where its tiles divide the problem, else a run-time instantiation of
-  // the header kernel with the caller's tiles
-  if (ring64_fits((int)M, (int)N, (int)K)) {
-    if (c_is_f32) return dispatch_ring64<float, bf16_t>(A, B, C, (int)M, (int)N, (int)K, st);
-    return dispatch_ring64<bf16_t, bf16_t>(A, B, C, (int)M, (int)N, (int)K, st);
-  }
-  TFK_REQUIRE(jit_gemm_supports(M, N, K), TF_ERR_UNSUPPORTED,
-              "tf_gemm: bf16 needs M %% 16 == 0, N %% 16 == 0, K %% 32 == 0 (got %lld, %lld, %lld)", (long long)M,
-              (long long)N, (long long)K);
-  return jit_gemm(A, B, C, dtype, c_is_f32 ? 0 : 1, M, N, K, tm, tn, tk, num_stages, pipeline_level, st);
+  // bf16: the same kernels with the bf16 MFMAs (every kernel of this file is a template of the
+  // operand type)
+  TFK_REQUIRE(K % 8 == 0, TF_ERR_UNSUPPORTED, "tf_gemm: K (%lld) must be a multiple of 8", (long long)K);
+  if (c_is_f32) return dispatch<float, bf16_t>(A, B, C, (int)M, (int)N, (int)K, st);
+  return dispatch<bf16_t, bf16_t>(A, B, C, (int)M, (int)N, (int)K, st);
 }

@@ -1,11 +1,13 @@
-// Host launchers that instantiate the header macro kernels (kernels/*_device.hpp) at run time
-// for shapes and element types the ahead-of-time kernels of this library have no instance of.
+// Host launcher that instantiates the header attention kernel (kernels/flash_attention_device.hpp)
+// at run time for head dimensions the ahead-of-time kernels of this library have no instance of.
 //
-// This is the reference's own launch path (src/kernels/gemm.cu:21-59,63-142,
-// src/kernels/fused_two_gemms.cu:35-63, src/kernels/flash_attn.cu:16-55,58-152): the whole
-// problem shape and the tile sizes become template arguments of a generated wrapper, which is
-// compiled once per distinct argument set (JitCompiler caches it in the process and on disk)
-// and launched on the caller's stream.  Here it is the fallback behind the tuned entry points.
+// This is the reference's own launch path (src/kernels/flash_attn.cu:16-55,58-152; the same for
+// its other ops, src/kernels/gemm.cu:21-59,63-142, src/kernels/fused_two_gemms.cu:35-63): the
+// whole problem shape and the tile sizes become template arguments of a generated wrapper, which
+// is compiled once per distinct argument set (JitCompiler caches it in the process and on disk)
+// and launched on the caller's stream.  Here it is the fallback behind the tuned attention entry
+// point; the GEMM and the fused op have ahead-of-time kernels for every shape and both element
+// types (their run-time instantiations are reached through tf_jit_compile / tf_jit_launch).
 #include <cmath>
 #include <cstring>
 #include <sstream>
@@ -21,8 +23,6 @@ namespace {
 using tilefusion::jit::JitCompiler;
 
 const char* kPrelude =
-    "#include \"kernels/gemm_device.hpp\"\n"
-    "#include \"kernels/fused_two_gemms_device.hpp\"\n"
     "#include \"kernels/flash_attention_device.hpp\"\n"
     "using namespace tilefusion;\n"
     "using namespace tilefusion::kernels;\n"
@@ -102,39 +102,6 @@ int jit_flash_attention(const void* Q, const void* K, const void* Vt, void* O, i
   void* args[] = {&Q, &K, &Vt, &O};
   return compile_and_launch(name.str(), src.str(), dim3((unsigned)(Lq / tq), (unsigned)(Dv / thv), (unsigned)batch),
                             wr * 64, lds, args, st);
-}
-
-bool jit_gemm_supports(int64_t M, int64_t N, int64_t K) { return M % 16 == 0 && N % 16 == 0 && K % 32 == 0; }
-
-int jit_gemm(const void* A, const void* B, void* C, int dtype, int c_kind, int64_t M, int64_t N, int64_t K, int tm,
-             int tn, int tk, int num_stages, int pipeline_level, hipStream_t st) {
-  // 2 x 2 wavefronts: 32 rows and 32 columns of C per workgroup at least
-  if (tm % 32 != 0 || M % tm != 0 || tm > 128) tm = pick_divisor(M, {128, 64, 32});
-  if (tn % 32 != 0 || N % tn != 0 || tn > 128) tn = pick_divisor(N, {128, 64, 32});
-  if (tk % 32 != 0 || K % tk != 0 || tk > 128) tk = pick_divisor(K, {64, 32});
-  int wr = 2, wc = 2;
-  if (tm == 0) { tm = pick_divisor(M, {16}); wr = 1; }
-  if (tn == 0) { tn = pick_divisor(N, {16}); wc = 1; }
-  TFK_REQUIRE(tm > 0 && tn > 0 && tk > 0, TF_ERR_UNSUPPORTED, "gemm: no legal tiling for M=%lld N=%lld K=%lld",
-              (long long)M, (long long)N, (long long)K);
-  if (pipeline_level > 0 && num_stages < 2) num_stages = 2;
-  const char* T = type_name(dtype);
-  const char* CT = c_kind == 0 ? "float" : T;
-  const char* entry =
-      pipeline_level == 0 ? "ke_gemm" : (pipeline_level == 1 ? "ke_gemm_level1_pipeline" : "ke_gemm_level2_pipeline");
-  std::ostringstream name, src;
-  name << "tf_gemm_" << (dtype == TF_DTYPE_BF16 ? "bf16_" : "f16_") << (c_kind == 0 ? "f32_" : "same_") << M << "_" << N
-       << "_" << K << "_" << tm << "_" << tn << "_" << tk << "_" << num_stages << "_" << pipeline_level << "_" << wr << wc;
-  src << kPrelude << "using Config = KeGemmTraits<" << T << ", " << CT << ", tl::RowMajor<" << wr << ", " << wc << ">, " << M
-      << ", " << N << ", " << K << ", " << tm << ", " << tn << ", " << tk << ", 32, " << num_stages << ", 64>;\n"
-      << "extern \"C\" __global__ __launch_bounds__(" << wr * wc * 64 << ") void " << name.str() << "(const " << T
-      << "* A, const " << T << "* B, " << CT << "* C) {\n  " << entry << "<" << T << ", " << CT
-      << ", Config>(A, B, C);\n}\n";
-  const int slots = pipeline_level > 0 ? num_stages : (num_stages >= 2 ? 2 : 1);
-  const unsigned lds = (unsigned)(tm * tk + tk * tn) * slots * 2u;
-  void* args[] = {&A, &B, &C};
-  return compile_and_launch(name.str(), src.str(), dim3((unsigned)(M / tm), (unsigned)(N / tn)), wr * wc * 64, lds, args,
-                            st);
 }
 
 }  // namespace tfk

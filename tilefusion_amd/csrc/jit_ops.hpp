@@ -1,5 +1,5 @@
-// Run-time instantiations of the header macro kernels, used behind the C ABI for shapes and
-// element types that have no ahead-of-time kernel (see jit_ops.cpp).
+// Run-time instantiation of the header attention kernel, used behind the C ABI for head dimensions
+// that have no ahead-of-time kernel (see jit_ops.cpp).
 #pragma once
 
 #include <cstdint>
@@ -7,11 +7,6 @@
 #include "common.hpp"
 
 namespace tfk {
-
-// c_kind: 0 = fp32 output, 1 = output in the input type
-bool jit_gemm_supports(int64_t M, int64_t N, int64_t K);
-int jit_gemm(const void* A, const void* B, void* C, int dtype, int c_kind, int64_t M, int64_t N, int64_t K, int tm,
-             int tn, int tk, int num_stages, int pipeline_level, hipStream_t st);
 
 // V must be handed over transposed ([batch, Dv, Lkv])
 bool jit_flash_attention_supports(int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int v_is_transposed);
