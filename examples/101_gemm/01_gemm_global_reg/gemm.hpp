@@ -17,23 +17,24 @@ struct GemmTraits {
   using WarpLayout = WarpLayout_;
   static constexpr int kWarpRows = tl::num_rows<WarpLayout>, kWarpCols = tl::num_cols<WarpLayout>;
   static constexpr int kThreads = tl::get_numel<WarpLayout> * WARP_SIZE;
-  static_assert(kTK % 32 == 0, "a register tile of fp16 operands is 32 deep in k");
+  using BaseShape = BaseTileShape<InType>;  // the 16 x 16 block one base tile covers
+  static_assert(kTK % BaseShape::kCols == 0, "a chunk is a whole number of base tiles deep");
 
   // A: rows of one C tile, all of K, walked in [kTM, kTK] chunks
   using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK>>;
   using IteratorA = TileIterator<GlobalA, TileShape<kTM, kTK>>;
-  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kTM / kWarpRows / 16, kTK / 32>>;
+  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kTM / kWarpRows / BaseShape::kRows, kTK / BaseShape::kCols>>;
   using ALoader = GlobalToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
 
   // B: column-major K x kTN
   using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kTN>>;
   using IteratorB = TileIterator<GlobalB, TileShape<kTK, kTN>>;
-  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kTN / kWarpCols / 16>>;
+  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / BaseShape::kRows, kTN / kWarpCols / BaseShape::kCols>>;
   using BLoader = GlobalToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
 
   // C: a [kTM, kTN] window of the row-major [kM, kN] output
   using GlobalC = GlobalTile<AccType, tl::RowMajor<kTM, kTN, kN>>;
-  using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kTM / kWarpRows / 16, kTN / kWarpCols / 16>>;
+  using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kTM / kWarpRows / BaseShape::kRows, kTN / kWarpCols / BaseShape::kCols>>;
   using CStorer = RegToGlobalStorer<GlobalC, RegC, WarpLayout>;
 };
 

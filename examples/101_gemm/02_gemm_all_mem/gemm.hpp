@@ -1,6 +1,6 @@
 // GEMM through all three memory levels (counterpart of examples/101_gemm/02_gemm_all_mem/
 // gemm.hpp): global -> LDS with GlobalToSharedLoader into swizzled SharedTiles, LDS ->
-// registers with SharedToRegLoader in MFMA fragment order, gemm() on the register tiles, and
+// registers with SharedToRegLoader in base-tile lane order, gemm() on the register tiles, and
 // the accumulator back to global memory.  One workgroup per [kTM, kTN] tile of C; K is walked
 // in kTK chunks through LDS and in kRK steps through registers.
 #pragma once
@@ -19,13 +19,14 @@ struct GemmTraits {
   using WarpLayout = WarpLayout_;
   static constexpr int kWarpRows = tl::num_rows<WarpLayout>, kWarpCols = tl::num_cols<WarpLayout>;
   static constexpr int kThreads = tl::get_numel<WarpLayout> * WARP_SIZE;
-  static_assert(kRK % 32 == 0 && kTK % kRK == 0, "kRK is a multiple of the 32-deep MFMA step and divides kTK");
+  using BaseShape = BaseTileShape<InType>;  // the 16 x 16 block one base tile covers
+  static_assert(kRK % BaseShape::kCols == 0 && kTK % kRK == 0, "kRK is whole base tiles and divides kTK");
 
   using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK>>;
   using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
   using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, /*swizzled=*/true, /*bytes=*/64>;
   using SIteratorA = STileIterator<SharedA, TileShape<kTM, kRK>>;
-  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kTM / kWarpRows / 16, kRK / 32>>;
+  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kTM / kWarpRows / BaseShape::kRows, kRK / BaseShape::kCols>>;
   using G2SLoaderA = GlobalToSharedLoader<SharedA, WarpLayout>;
   using S2RLoaderA = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
 
@@ -33,12 +34,12 @@ struct GemmTraits {
   using GIteratorB = GTileIterator<GlobalB, TileShape<kTK, kTN>>;
   using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, true, 64>;
   using SIteratorB = STileIterator<SharedB, TileShape<kRK, kTN>>;
-  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kRK / 32, kTN / kWarpCols / 16>>;
+  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kRK / BaseShape::kRows, kTN / kWarpCols / BaseShape::kCols>>;
   using G2SLoaderB = GlobalToSharedLoader<SharedB, WarpLayout>;
   using S2RLoaderB = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
 
   using GlobalC = GlobalTile<AccType, tl::RowMajor<kTM, kTN, kN>>;
-  using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kTM / kWarpRows / 16, kTN / kWarpCols / 16>>;
+  using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kTM / kWarpRows / BaseShape::kRows, kTN / kWarpCols / BaseShape::kCols>>;
   using R2GStorerC = RegToGlobalStorer<GlobalC, RegC, WarpLayout>;
 
   static constexpr int kSharedBytes = (SharedA::kNumel + SharedB::kNumel) * (int)sizeof(InType);

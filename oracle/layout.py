@@ -235,3 +235,28 @@ def mfma_16x16x32_ab(lane, t):
 
 def mfma_16x16x32_c(lane, r):
     return 4 * (lane // 16) + r, lane % 16
+
+
+# --- base-tile lane maps of the tile API on a 64-lane wavefront (the reference's are for the
+# 32-thread mma.m16n8k16 fragments, include/cell/copy/global_to_register.hpp:40-55).  A base tile
+# covers the reference's 16 x 16 block (include/types/base.hpp:62-68); `per_lane` is 4 for it and
+# 8 for the wide 16 x 32 / 32 x 16 operand block. ---------------------------------------------
+
+def base_tile_coord(lane, e, row_major, per_lane=4):
+    """(row, col) inside the block of per-lane element e: a row-major base tile gives lane l the
+    columns per_lane*(l//16).. of row l%16, a column-major one the rows per_lane*(l//16).. of
+    column l%16."""
+    if row_major:
+        return lane % 16, per_lane * (lane // 16) + e
+    return per_lane * (lane // 16) + e, lane % 16
+
+
+def base_tile_shape(row_major, per_lane=4):
+    """(rows, cols) of the block one base tile covers."""
+    return (16, 4 * per_lane) if row_major else (4 * per_lane, 16)
+
+
+def paired_k_assignment(lane, e):
+    """k index (0..31) that element e (0..7) of the 8-element operand fragment built from two
+    square base tiles adjacent in k carries: elements 0-3 come from the first tile."""
+    return 16 * (e // 4) + 4 * (lane // 16) + e % 4

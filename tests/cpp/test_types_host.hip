@@ -66,8 +66,16 @@ static_assert(wbt<__half, 128, 128, RM, 64, 8, 64, 8, 8>() && wbt<__half, 128, 1
 static_assert(wbt<float, 128, 128, RM, 64, 8, 32, 8, 8>() && wbt<__half, 64, 16, RM, 64, 32, 16, 32, 2>());
 
 // ---- base tiles ------------------------------------------------------------------------------
-static_assert(BaseTileShape<__half>::kRows == 16 && BaseTileShape<__half>::kCols == 32 && BaseTileShape<float>::kCols == 16);
-static_assert(BaseTileRowMajor<__half>::kNumel == 8 && BaseTileColMajor<__half>::kNumel == 8 && BaseTileRowMajor<float>::kNumel == 4);
+// square base tiles for every type (include/types/base.hpp:62-68), 4 elements per lane on 64 lanes
+static_assert(BaseTileShape<__half>::kRows == 16 && BaseTileShape<__half>::kCols == 16 && BaseTileShape<float>::kRows == 16 &&
+              BaseTileShape<float>::kCols == 16 && BaseTileShape<__bfloat16>::kNumel == 256);
+static_assert(BaseTileRowMajor<__half>::kNumel == 4 && BaseTileColMajor<__half>::kNumel == 4 && BaseTileRowMajor<float>::kNumel == 4 &&
+              BaseTileRowMajor<float>::kNumel * WARP_SIZE == BaseTileShape<float>::kNumel);
+static_assert(BaseTileTraits<BaseTileRowMajor<float>>::kIsRowMajor && !BaseTileTraits<BaseTileColMajor<__half>>::kIsRowMajor &&
+              BaseTileTraits<BaseTileRowMajor<__half>>::kRows == 16 && BaseTileTraits<BaseTileRowMajor<__half>>::kCols == 16);
+static_assert(WideBaseTileShape<__half>::kCols == 32 && WideBaseTileRowMajor<__half>::kNumel == 8 &&
+              BaseTileTraits<WideBaseTileRowMajor<__half>>::kCols == 32 && BaseTileTraits<WideBaseTileColMajor<__half>>::kRows == 32 &&
+              BaseTileTraits<WideBaseTileColMajor<__half>>::kCols == 16);
 static_assert(dim_size<0, TileShape<128, 32>> == 128 && dim_size<1, TileShape<128, 32>> == 32 && get_numel<TileShape<2, 3, 4>> == 24);
 
 int main() {

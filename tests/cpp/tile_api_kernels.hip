@@ -68,8 +68,12 @@ TT_API void tt_g2s_shape(int variant, int* rows, int* cols, int* elem_bytes, int
 
 // ---- 2. swizzled and plain LDS tiles give identical register fragments, and an accumulator
 //         tile survives register -> LDS -> global (test_swizzled_copy.cu:27-94, test_s2r_copy.cu) --
-template <typename WarpLayout, int kRows, int kCols, int kChunk, int kBytes>
+template <typename WarpLayout, int kRows, int kCols, int kChunk, int kBytes, bool kWide>
 __global__ void k_swizzled_fragments(const __half* a_in, const __half* b_in, int* mismatches) {
+  // kWide: 16 x 32 operand base tiles (8 elements per lane), else the square 16 x 16 ones (4)
+  constexpr int kDepth = kWide ? 32 : 16, kPerLane = kWide ? 8 : 4;
+  using BaseA = std::conditional_t<kWide, RegTile<__half, tl::RowMajor<1, 8>>, BaseTileRowMajor<__half>>;
+  using BaseB = std::conditional_t<kWide, RegTile<__half, tl::ColMajor<8, 1>>, BaseTileColMajor<__half>>;
   extern __shared__ __attribute__((aligned(16))) unsigned char buf[];
   __half* base = reinterpret_cast<__half*>(buf);
   using GlobalA = GlobalTile<__half, tl::RowMajor<kRows, kCols>>;
@@ -91,8 +95,8 @@ __global__ void k_swizzled_fragments(const __half* a_in, const __half* b_in, int
   __copy_async();
   __syncthreads();
   constexpr int kWR = tl::num_rows<WarpLayout>, kWC = tl::num_cols<WarpLayout>;
-  using RegA = RegTile<BaseTileRowMajor<__half>, tl::RowMajor<kRows / kWR / 16, kChunk / 32>>;
-  using RegB = RegTile<BaseTileColMajor<__half>, tl::ColMajor<kChunk / 32, kRows / kWC / 16>>;
+  using RegA = RegTile<BaseA, tl::RowMajor<kRows / kWR / 16, kChunk / kDepth>>;
+  using RegB = RegTile<BaseB, tl::ColMajor<kChunk / kDepth, kRows / kWC / 16>>;
   using IterA0 = STileIterator<SA0, TileShape<kRows, kChunk>>;
   using IterA1 = STileIterator<SA1, TileShape<kRows, kChunk>>;
   using IterB0 = STileIterator<SB0, TileShape<kChunk, kRows>>;
@@ -113,47 +117,59 @@ __global__ void k_swizzled_fragments(const __half* a_in, const __half* b_in, int
     lb(ib1(k), rb1);
     const __half* p0 = ra0.data()[0].data();
     const __half* p1 = ra1.data()[0].data();
-    for (int e = 0; e < RegA::kNumel * 8; ++e) bad += (__half2float(p0[e]) != __half2float(p1[e]));
+    for (int e = 0; e < RegA::kNumel * kPerLane; ++e) bad += (__half2float(p0[e]) != __half2float(p1[e]));
     const __half* q0 = rb0.data()[0].data();
     const __half* q1 = rb1.data()[0].data();
-    for (int e = 0; e < RegB::kNumel * 8; ++e) bad += (__half2float(q0[e]) != __half2float(q1[e]));
+    for (int e = 0; e < RegB::kNumel * kPerLane; ++e) bad += (__half2float(q0[e]) != __half2float(q1[e]));
     // and the fragment really is the documented block of the source: element 0 of base tile (0,0)
     const int lane = threadIdx.x % WARP_SIZE;
     const int wr = warp::warp_row_id<WarpLayout>();
-    const float want = __half2float(a_in[(wr * (kRows / kWR) + lane % 16) * kCols + k * kChunk + 8 * (lane / 16)]);
+    const float want = __half2float(a_in[(wr * (kRows / kWR) + lane % 16) * kCols + k * kChunk + kPerLane * (lane / 16)]);
     bad += (__half2float(p0[0]) != want);
+    // same for B (a column-major [kCols, kRows] matrix: element (r, c) at c * kCols + r)
+    const int wc = warp::warp_col_id<WarpLayout>();
+    const float want_b = __half2float(b_in[(wc * (kRows / kWC) + lane % 16) * kCols + k * kChunk + kPerLane * (lane / 16)]);
+    bad += (__half2float(q0[0]) != want_b);
   }
   if (bad) atomicAdd(mismatches, bad);
 }
-TT_API int tt_swizzled_fragments(int variant, const void* a, const void* b, int* mismatches) {
-  const __half* pa = static_cast<const __half*>(a);
-  const __half* pb = static_cast<const __half*>(b);
-  switch (variant) {
+template <bool kWide>
+static int run_swizzled_fragments(int shape, const __half* pa, const __half* pb, int* mismatches) {
+  switch (shape) {
     case 0:
-      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<1, 1>, 64, 64, 32, 128>), dim3(1), dim3(64), 4 * 64 * 64 * 2, 0, pa, pb, mismatches);
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<1, 1>, 64, 64, 32, 128, kWide>), dim3(1), dim3(64), 4 * 64 * 64 * 2, 0, pa, pb, mismatches);
       break;
     case 1:
-      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<2, 2>, 128, 128, 64, 128>), dim3(1), dim3(256), 4 * 128 * 128 * 2, 0, pa, pb, mismatches);
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<2, 2>, 128, 128, 64, 128, kWide>), dim3(1), dim3(256), 4 * 128 * 128 * 2, 0, pa, pb, mismatches);
       break;
     case 2:
-      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<2, 2>, 64, 128, 32, 64>), dim3(1), dim3(256), 4 * 64 * 128 * 2, 0, pa, pb, mismatches);
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<2, 2>, 64, 128, 32, 64, kWide>), dim3(1), dim3(256), 4 * 64 * 128 * 2, 0, pa, pb, mismatches);
       break;
     case 3:
-      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<4, 1>, 64, 64, 64, 64>), dim3(1), dim3(256), 4 * 64 * 64 * 2, 0, pa, pb, mismatches);
+      hipLaunchKernelGGL((k_swizzled_fragments<tl::RowMajor<4, 1>, 64, 64, 64, 64, kWide>), dim3(1), dim3(256), 4 * 64 * 64 * 2, 0, pa, pb, mismatches);
       break;
     default: return -1;
   }
   return launch_status();
 }
+// variants 0-3: wide operand tiles, 4-7: the same shapes with square base tiles
+TT_API int tt_swizzled_fragments(int variant, const void* a, const void* b, int* mismatches) {
+  const __half* pa = static_cast<const __half*>(a);
+  const __half* pb = static_cast<const __half*>(b);
+  return variant < 4 ? run_swizzled_fragments<true>(variant, pa, pb, mismatches)
+                     : run_swizzled_fragments<false>(variant - 4, pa, pb, mismatches);
+}
 
-template <typename WarpLayout, int kRows, int kCols>
+template <typename WarpLayout, int kRows, int kCols, bool kColTiles>
 __global__ void k_acc_roundtrip(const float* in, float* out_direct, float* out_via_lds, __half* out_half) {
   extern __shared__ __attribute__((aligned(16))) unsigned char buf[];
   constexpr int kWR = tl::num_rows<WarpLayout>, kWC = tl::num_cols<WarpLayout>;
   using Global = GlobalTile<float, tl::RowMajor<kRows, kCols>>;
   using GlobalH = GlobalTile<__half, tl::RowMajor<kRows, kCols>>;
-  using Reg = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kRows / kWR / 16, kCols / kWC / 16>>;
-  using RegH = RegTile<BaseTileAccRowMajor<__half>, tl::RowMajor<kRows / kWR / 16, kCols / kWC / 16>>;
+  using Reg = RegTile<std::conditional_t<kColTiles, BaseTileColMajor<float>, BaseTileRowMajor<float>>,
+                      tl::RowMajor<kRows / kWR / 16, kCols / kWC / 16>>;
+  using RegH = RegTile<std::conditional_t<kColTiles, BaseTileColMajor<__half>, BaseTileRowMajor<__half>>,
+                       tl::RowMajor<kRows / kWR / 16, kCols / kWC / 16>>;
   using Shared = SharedTile<float, tl::RowMajor<kRows, kCols>, true, 128>;
   Global g_in(in), g_direct(out_direct), g_lds(out_via_lds);
   GlobalH g_half(out_half);
@@ -181,10 +197,17 @@ TT_API int tt_acc_roundtrip(int variant, const void* in, void* out_direct, void*
   __half* ph = static_cast<__half*>(out_half);
   switch (variant) {
     case 0:
-      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<1, 1>, 32, 64>), dim3(1), dim3(64), 32 * 64 * 4, 0, pi, po, pl, ph);
+      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<1, 1>, 32, 64, false>), dim3(1), dim3(64), 32 * 64 * 4, 0, pi, po, pl, ph);
       break;
     case 1:
-      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<2, 2>, 128, 64>), dim3(1), dim3(256), 128 * 64 * 4, 0, pi, po, pl, ph);
+      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<2, 2>, 128, 64, false>), dim3(1), dim3(256), 128 * 64 * 4, 0, pi, po, pl, ph);
+      break;
+    // the same shapes held as column-major base tiles (a lane owns part of a column)
+    case 2:
+      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<1, 1>, 32, 64, true>), dim3(1), dim3(64), 32 * 64 * 4, 0, pi, po, pl, ph);
+      break;
+    case 3:
+      hipLaunchKernelGGL((k_acc_roundtrip<tl::RowMajor<2, 2>, 128, 64, true>), dim3(1), dim3(256), 128 * 64 * 4, 0, pi, po, pl, ph);
       break;
     default: return -1;
   }
@@ -192,22 +215,26 @@ TT_API int tt_acc_roundtrip(int variant, const void* in, void* out_direct, void*
 }
 
 // ---- 3. the README example: GEMM with global -> register loaders only (README.md:56-112,
-//         examples/101_gemm/01_gemm_global_reg/gemm.hpp:62-95) with the consistent tile shapes ----
+//         examples/101_gemm/01_gemm_global_reg/gemm.hpp:62-95); the tile counts are the reference's
+//         formulas over the square BaseTileShape (gemm.hpp:19-56 there), the accumulator is the
+//         BaseTileRowMajor<float> tile the README declares ----
 namespace readme {
 using InType = __half;
 using AccType = float;
 using WarpLayout = tl::RowMajor<2, 2>;
 constexpr int kM = 128, kN = 64, kK = 256, kTK = 32;
+using BaseShape = BaseTileShape<InType>;
+constexpr int kWarpPerRow = tl::num_rows<WarpLayout>, kWarpPerCol = tl::num_cols<WarpLayout>;
 using GlobalA = GlobalTile<InType, tl::RowMajor<kM, kK>>;
 using IteratorA = TileIterator<GlobalA, TileShape<kM, kTK>>;
-using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kM / 2 / 16, kTK / 32>>;
+using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kM / kWarpPerRow / BaseShape::kRows, kTK / BaseShape::kCols>>;
 using ALoader = GlobalToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
 using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kN>>;
 using IteratorB = TileIterator<GlobalB, TileShape<kTK, kN>>;
-using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kN / 2 / 16>>;
+using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / BaseShape::kRows, kN / kWarpPerCol / BaseShape::kCols>>;
 using BLoader = GlobalToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
 using GlobalC = GlobalTile<AccType, tl::RowMajor<kM, kN>>;
-using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kM / 2 / 16, kN / 2 / 16>>;
+using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kM / kWarpPerRow / BaseShape::kRows, kN / kWarpPerCol / BaseShape::kCols>>;
 using CStorer = RegToGlobalStorer<GlobalC, RegC, WarpLayout>;
 
 __global__ void simple_gemm(const InType* dA, const InType* dB, AccType* dC) {
@@ -239,18 +266,23 @@ TT_API int tt_readme_gemm(const void* a, const void* b, void* c) {
 // ---- 3b. the same GEMM with the other MMA atoms: bf16 inputs, and fp16 inputs with an fp16
 //          accumulator tile (include/cell/compute/gemm.hpp:63-150 in the reference) -------------
 namespace atoms {
-template <typename InType, typename AccType>
+// kWide: wide 16 x 32 operand tiles; kColAcc: column-major accumulator base tiles; kTK = 48 walks
+// an odd number of square base tiles per chunk (one 16x16x32 and one 16x16x16 instruction)
+template <typename InType, typename AccType, bool kWide, bool kColAcc, int kTK>
 __global__ void gemm_atom(const InType* dA, const InType* dB, AccType* dC) {
   using WarpLayout = tl::RowMajor<2, 2>;
-  constexpr int kM = 128, kN = 64, kK = 256, kTK = 32;
+  constexpr int kM = 128, kN = 64, kK = 192, kDepth = kWide ? 32 : 16;
+  using BaseA = std::conditional_t<kWide, RegTile<InType, tl::RowMajor<1, 8>>, BaseTileRowMajor<InType>>;
+  using BaseB = std::conditional_t<kWide, RegTile<InType, tl::ColMajor<8, 1>>, BaseTileColMajor<InType>>;
+  using BaseC = std::conditional_t<kColAcc, BaseTileColMajor<AccType>, BaseTileRowMajor<AccType>>;
   using GlobalA = GlobalTile<InType, tl::RowMajor<kM, kK>>;
   using IteratorA = TileIterator<GlobalA, TileShape<kM, kTK>>;
-  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kM / 2 / 16, kTK / 32>>;
+  using RegA = RegTile<BaseA, tl::RowMajor<kM / 2 / 16, kTK / kDepth>>;
   using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kN>>;
   using IteratorB = TileIterator<GlobalB, TileShape<kTK, kN>>;
-  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kN / 2 / 16>>;
+  using RegB = RegTile<BaseB, tl::ColMajor<kTK / kDepth, kN / 2 / 16>>;
   using GlobalC = GlobalTile<AccType, tl::RowMajor<kM, kN>>;
-  using RegC = RegTile<BaseTileAccRowMajor<AccType>, tl::RowMajor<kM / 2 / 16, kN / 2 / 16>>;
+  using RegC = RegTile<BaseC, tl::RowMajor<kM / 2 / 16, kN / 2 / 16>>;
   IteratorA gAs(dA);
   IteratorB gBs(dB);
   RegA rA;
@@ -267,14 +299,63 @@ __global__ void gemm_atom(const InType* dA, const InType* dB, AccType* dC) {
   RegToGlobalStorer<GlobalC, RegC, WarpLayout> storer_c;
   storer_c(acc, gC);
 }
+// MmaAtom used directly on single base tiles: C[16,16] += A[16,16] * B[16,16] (one wavefront)
+template <typename InType>
+__global__ void single_atom(const InType* dA, const InType* dB, float* dC) {
+  using Atom = compute::MmaAtom<InType, InType, float, compute::MMA_ATOM_16x16x16>;
+  using WarpLayout = tl::RowMajor<1, 1>;
+  using RegA = RegTile<typename Atom::BaseTileA, tl::RowMajor<1, 1>>;
+  using RegB = RegTile<typename Atom::BaseTileB, tl::ColMajor<1, 1>>;
+  using RegC = RegTile<typename Atom::BaseTileC, tl::RowMajor<1, 1>>;
+  using GlobalA = GlobalTile<InType, tl::RowMajor<16, 16>>;
+  using GlobalB = GlobalTile<InType, tl::ColMajor<16, 16>>;
+  using GlobalC = GlobalTile<float, tl::RowMajor<16, 16>>;
+  GlobalA gA(dA);
+  GlobalB gB(dB);
+  GlobalC gC(dC);
+  RegA rA;
+  RegB rB;
+  RegC rC;
+  GlobalToRegLoader<RegA, WarpLayout, WarpReuse::kCont> la;
+  GlobalToRegLoader<RegB, WarpLayout, WarpReuse::kCont> lb;
+  la(gA, rA);
+  lb(gB, rB);
+  Atom mma;
+  mma(rA(0, 0), rB(0, 0), rC(0, 0));
+  RegToGlobalStorer<GlobalC, RegC, WarpLayout> sc;
+  sc(rC, gC);
+}
 }  // namespace atoms
+// variant: 0 bf16 -> fp32, 1 fp16 -> fp16 accumulator, 2 fp16 -> fp32 with a column-major accumulator,
+// 3 fp16 -> fp32 with an odd base-tile count per chunk, 4 bf16 odd count; +8: the same with wide
+// operand tiles (variants 8, 9, 10).  A [128, 192], B [192, 64] column-major, C [128, 64].
 TT_API int tt_atom_gemm(int variant, const void* a, const void* b, void* c) {
+  const auto* ha = static_cast<const __half*>(a);
+  const auto* hb = static_cast<const __half*>(b);
+  const auto* ba = static_cast<const __bfloat16*>(a);
+  const auto* bb = static_cast<const __bfloat16*>(b);
+  const dim3 g(1), t(256);
+  switch (variant) {
+    case 0: hipLaunchKernelGGL((atoms::gemm_atom<__bfloat16, float, false, false, 32>), g, t, 0, 0, ba, bb, static_cast<float*>(c)); break;
+    case 1: hipLaunchKernelGGL((atoms::gemm_atom<__half, __half, false, false, 32>), g, t, 0, 0, ha, hb, static_cast<__half*>(c)); break;
+    case 2: hipLaunchKernelGGL((atoms::gemm_atom<__half, float, false, true, 32>), g, t, 0, 0, ha, hb, static_cast<float*>(c)); break;
+    case 3: hipLaunchKernelGGL((atoms::gemm_atom<__half, float, false, false, 48>), g, t, 0, 0, ha, hb, static_cast<float*>(c)); break;
+    case 4: hipLaunchKernelGGL((atoms::gemm_atom<__bfloat16, float, false, true, 48>), g, t, 0, 0, ba, bb, static_cast<float*>(c)); break;
+    case 8: hipLaunchKernelGGL((atoms::gemm_atom<__bfloat16, float, true, false, 32>), g, t, 0, 0, ba, bb, static_cast<float*>(c)); break;
+    case 9: hipLaunchKernelGGL((atoms::gemm_atom<__half, __half, true, false, 64>), g, t, 0, 0, ha, hb, static_cast<__half*>(c)); break;
+    case 10: hipLaunchKernelGGL((atoms::gemm_atom<__half, float, true, true, 32>), g, t, 0, 0, ha, hb, static_cast<float*>(c)); break;
+    default: return -1;
+  }
+  return launch_status();
+}
+// one MmaAtom on one base tile each: variant 0 fp16, 1 bf16
+TT_API int tt_single_atom(int variant, const void* a, const void* b, void* c) {
   if (variant == 0)
-    hipLaunchKernelGGL((atoms::gemm_atom<__bfloat16, float>), dim3(1), dim3(256), 0, 0, static_cast<const __bfloat16*>(a),
-                       static_cast<const __bfloat16*>(b), static_cast<float*>(c));
+    hipLaunchKernelGGL((atoms::single_atom<__half>), dim3(1), dim3(64), 0, 0, static_cast<const __half*>(a),
+                       static_cast<const __half*>(b), static_cast<float*>(c));
   else if (variant == 1)
-    hipLaunchKernelGGL((atoms::gemm_atom<__half, __half>), dim3(1), dim3(256), 0, 0, static_cast<const __half*>(a),
-                       static_cast<const __half*>(b), static_cast<__half*>(c));
+    hipLaunchKernelGGL((atoms::single_atom<__bfloat16>), dim3(1), dim3(64), 0, 0, static_cast<const __bfloat16*>(a),
+                       static_cast<const __bfloat16*>(b), static_cast<float*>(c));
   else
     return -1;
   return launch_status();
@@ -312,14 +393,16 @@ TT_API void tt_ke_gemm_shape(int variant, int* m, int* n, int* k, int* c_is_half
 
 // ---- 5. reduce / broadcast / map / mask on an accumulator tile (print-only in the reference:
 //         tests/cpp/cell/test_reduce.cu, test_broadcast.cu, test_flash_attn.cu) ------------------
-template <typename WarpLayout, int kRows, int kCols>
+template <typename WarpLayout, int kRows, int kCols, int kVecCols>
 __global__ void k_softmax_pieces(const float* in, float* row_max, float* row_sum, float* out, int row_offset,
                                  int col_offset) {
   constexpr int kWR = tl::num_rows<WarpLayout>;
   static_assert(tl::num_cols<WarpLayout> == 1, "rows must not be split across wavefronts");
   using Global = GlobalTile<float, tl::RowMajor<kRows, kCols>>;
   using Reg = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kRows / kWR / 16, kCols / 16>>;
-  using Vec = RegTile<float, tl::RowMajor<Reg::kRows, 4>>;
+  // one row per lane and base-tile row; kVecCols = 2 is how kernels written for the reference
+  // declare the vector (every column then holds the same value)
+  using Vec = RegTile<float, tl::RowMajor<Reg::kRows, kVecCols>>;
   Global g_in(in), g_out(out);
   Reg t;
   GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;
@@ -343,13 +426,12 @@ __global__ void k_softmax_pieces(const float* in, float* row_max, float* row_sum
   r2g(t, g_out);
   const int lane = threadIdx.x % WARP_SIZE;
   const int wrow = warp::warp_row_id<WarpLayout>() * (kRows / kWR);
-  if (lane % 16 == 0) {
-    for (int i = 0; i < Reg::kRows; ++i)
-      for (int r = 0; r < 4; ++r) {
-        row_max[wrow + 16 * i + 4 * (lane / 16) + r] = vmax(i, r);
-        row_sum[wrow + 16 * i + 4 * (lane / 16) + r] = vsum(i, r);
-      }
-  }
+  // every one of the four lanes that share a row must hold the result: lane group g writes rows with row % 4 == g
+  for (int i = 0; i < Reg::kRows; ++i)
+    if ((lane % 16) % 4 == lane / 16) {
+      row_max[wrow + 16 * i + lane % 16] = vmax(i, kVecCols - 1);
+      row_sum[wrow + 16 * i + lane % 16] = vsum(i, kVecCols - 1);
+    }
 }
 TT_API int tt_softmax_pieces(int variant, const void* in, void* row_max, void* row_sum, void* out, int row_offset,
                              int col_offset) {
@@ -357,13 +439,13 @@ TT_API int tt_softmax_pieces(int variant, const void* in, void* row_max, void* r
   float *pm = static_cast<float*>(row_max), *ps = static_cast<float*>(row_sum), *po = static_cast<float*>(out);
   switch (variant) {
     case 0:
-      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<1, 1>, 16, 16>), dim3(1), dim3(64), 0, 0, pi, pm, ps, po, row_offset, col_offset);
+      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<1, 1>, 16, 16, 1>), dim3(1), dim3(64), 0, 0, pi, pm, ps, po, row_offset, col_offset);
       break;
     case 1:
-      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<1, 1>, 32, 64>), dim3(1), dim3(64), 0, 0, pi, pm, ps, po, row_offset, col_offset);
+      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<1, 1>, 32, 64, 2>), dim3(1), dim3(64), 0, 0, pi, pm, ps, po, row_offset, col_offset);
       break;
     case 2:
-      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<4, 1>, 128, 128>), dim3(1), dim3(256), 0, 0, pi, pm, ps, po, row_offset, col_offset);
+      hipLaunchKernelGGL((k_softmax_pieces<tl::RowMajor<4, 1>, 128, 128, 1>), dim3(1), dim3(256), 0, 0, pi, pm, ps, po, row_offset, col_offset);
       break;
     default: return -1;
   }
@@ -409,8 +491,8 @@ __global__ __launch_bounds__(Traits::kThreads) void k_ke_flash(const __half* q, 
 }
 template <typename WarpLayout, int B, int M, int N, int K, int P, int TM, int TN, int TK, int TP, bool kCausal>
 static int run_ke_flash(const void* q, const void* k, const void* v, void* o) {
-  // softmax scale 1/sqrt(K): K is 64 or 128 in every variant below
-  constexpr double kScale = K == 128 ? 0.08838834764831845 : 0.125;
+  // softmax scale 1/sqrt(K): K is 128, 64 or 96 in the variants below
+  constexpr double kScale = K == 128 ? 0.08838834764831845 : K == 64 ? 0.125 : 0.10206207261596575;
   using Traits = kernels::FlashAttentionTraits<__half, float, __half, TileShape<M, N, K, P>, TileShape<TM, TN, TK, TP>,
                                                WarpLayout, kScale, kCausal>;
   auto kern = k_ke_flash<Traits>;
@@ -420,8 +502,9 @@ static int run_ke_flash(const void* q, const void* k, const void* v, void* o) {
                      static_cast<__half*>(o));
   return launch_status();
 }
-static const int kFlashShapes[6][6] = {{1, 64, 128, 128, 128, 0},  {1, 128, 128, 128, 128, 1}, {2, 256, 512, 128, 128, 0},
-                                       {2, 512, 512, 64, 64, 1},   {1, 128, 256, 64, 128, 0},  {3, 256, 256, 128, 64, 1}};
+static const int kFlashShapes[7][6] = {{1, 64, 128, 128, 128, 0},  {1, 128, 128, 128, 128, 1}, {2, 256, 512, 128, 128, 0},
+                                       {2, 512, 512, 64, 64, 1},   {1, 128, 256, 64, 128, 0},  {3, 256, 256, 128, 64, 1},
+                                       {2, 64, 128, 96, 64, 1}};
 TT_API int tt_ke_flash(int variant, const void* q, const void* k, const void* v, void* o) {
   switch (variant) {
     case 0: return run_ke_flash<tl::RowMajor<4, 1>, 1, 64, 128, 128, 128, 64, 128, 128, 128, false>(q, k, v, o);
@@ -430,6 +513,8 @@ TT_API int tt_ke_flash(int variant, const void* q, const void* k, const void* v,
     case 3: return run_ke_flash<tl::RowMajor<4, 1>, 2, 512, 512, 64, 64, 128, 64, 64, 64, true>(q, k, v, o);
     case 4: return run_ke_flash<tl::RowMajor<2, 1>, 1, 128, 256, 64, 128, 32, 128, 32, 64, false>(q, k, v, o);
     case 5: return run_ke_flash<tl::RowMajor<1, 1>, 3, 256, 256, 128, 64, 16, 32, 64, 32, true>(q, k, v, o);
+    // head dimension 96 walked in three 32-deep chunks (Q reloaded per key tile)
+    case 6: return run_ke_flash<tl::RowMajor<2, 1>, 2, 64, 128, 96, 64, 32, 64, 32, 64, true>(q, k, v, o);
     default: return -1;
   }
 }
@@ -608,6 +693,7 @@ __global__ void k_warp_helpers(long long* out) {
     out[wid * 6 + 5] = Exec::col_exec_count();
   }
 }
+struct Base16x16 { static constexpr int kRows = 16, kCols = 16; };
 struct Base16x32 { static constexpr int kRows = 16, kCols = 32; };
 struct Base32x16 { static constexpr int kRows = 32, kCols = 16; };
 template <typename WarpLayout, typename Tile, typename BaseShape>
@@ -626,6 +712,8 @@ TT_API int tt_warp_helpers(int layout, int mode, long long* out) {
     case 0: return run_warp_helpers<tl::RowMajor<2, 2>, GlobalTile<__half, tl::RowMajor<128, 256, 512>>, Base16x32>(mode, out);
     case 1: return run_warp_helpers<tl::RowMajor<4, 1>, GlobalTile<__half, tl::RowMajor<128, 64>>, Base16x32>(mode, out);
     case 2: return run_warp_helpers<tl::ColMajor<2, 2>, GlobalTile<__half, tl::ColMajor<128, 64, 256>>, Base32x16>(mode, out);
+    // layout 3: as layout 0 with square 16 x 16 base tiles
+    case 3: return run_warp_helpers<tl::RowMajor<2, 2>, GlobalTile<__half, tl::RowMajor<128, 256, 512>>, Base16x16>(mode, out);
     default: return -1;
   }
 }
@@ -733,7 +821,7 @@ __global__ void k_functors(const float* xin, const float* yin, float* out_add, f
   using WarpLayout = tl::RowMajor<2, 1>;
   using Global = GlobalTile<float, tl::RowMajor<64, 32>>;
   using Reg = RegTile<BaseTileRowMajor<float>, tl::RowMajor<2, 2>>;
-  using Vec = RegTile<float, tl::RowMajor<Reg::kRows, 4>>;
+  using Vec = RegTile<float, tl::RowMajor<Reg::kRows, 1>>;
   Global gx(xin), gy(yin);
   Reg x, y, t, one;
   GlobalToRegLoader<Reg, WarpLayout, WarpReuse::kCont> g2r;

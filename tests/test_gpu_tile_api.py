@@ -37,6 +37,7 @@ def lib():
     lib.tt_acc_roundtrip.argtypes = [_i, _vp, _vp, _vp, _vp]
     lib.tt_readme_gemm.argtypes = [_vp, _vp, _vp]
     lib.tt_atom_gemm.argtypes = [_i, _vp, _vp, _vp]
+    lib.tt_single_atom.argtypes = [_i, _vp, _vp, _vp]
     lib.tt_ke_gemm.argtypes = [_i, _vp, _vp, _vp]
     lib.tt_ke_gemm_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 4
     lib.tt_softmax_pieces.argtypes = [_i, _vp, _vp, _vp, _vp, _i, _i]
@@ -69,8 +70,11 @@ def test_global_shared_roundtrip_is_exact(lib, variant):
     assert torch.equal(src, dst)
 
 
-@pytest.mark.parametrize("variant,rows,cols", [(0, 64, 64), (1, 128, 128), (2, 64, 128), (3, 64, 64)])
-def test_swizzled_and_plain_lds_give_identical_fragments(lib, variant, rows, cols):
+@pytest.mark.parametrize("wide", [True, False])
+@pytest.mark.parametrize("shape,rows,cols", [(0, 64, 64), (1, 128, 128), (2, 64, 128), (3, 64, 64)])
+def test_swizzled_and_plain_lds_give_identical_fragments(lib, wide, shape, rows, cols):
+    # wide 16 x 32 operand base tiles (variants 0-3) and the square 16 x 16 ones (4-7)
+    variant = shape if wide else shape + 4
     a = (torch.arange(rows * cols) % 2048).half().to(DEV)
     b = ((torch.arange(rows * cols) * 7) % 2048).half().to(DEV)
     bad = torch.zeros(1, dtype=torch.int32, device=DEV)
@@ -78,8 +82,9 @@ def test_swizzled_and_plain_lds_give_identical_fragments(lib, variant, rows, col
     assert int(bad.item()) == 0
 
 
-@pytest.mark.parametrize("variant,rows,cols", [(0, 32, 64), (1, 128, 64)])
+@pytest.mark.parametrize("variant,rows,cols", [(0, 32, 64), (1, 128, 64), (2, 32, 64), (3, 128, 64)])
 def test_accumulator_tile_roundtrips(lib, variant, rows, cols):
+    # variants 0-1 hold the tile as row-major base tiles, 2-3 as column-major ones
     src = (torch.arange(rows * cols) % 2048).float().to(DEV)
     direct, via_lds = torch.full_like(src, -1), torch.full_like(src, -1)
     half = torch.full((rows * cols,), -1, dtype=torch.float16, device=DEV)
@@ -104,19 +109,57 @@ def test_readme_example_gemm(lib):
     assert torch.equal(c.cpu(), N.gemm_ref(a, b))
 
 
-def test_other_mma_atoms(lib):
-    # bf16 x bf16 -> fp32, and fp16 x fp16 with an fp16 accumulator tile (rounded once per atom)
-    a, b = oracle.make_c1_gemm_inputs()
-    ref = N.gemm_ref(a.bfloat16(), b.bfloat16())
+def test_readme_example_gemm_is_exact_for_each_k_chunk(lib):
+    # a wrong k assignment between the A and B fragments shows when only one 16-wide k block of
+    # the 256 is non-zero: every such block must give the exact partial product
+    g = torch.Generator().manual_seed(2)
     c = torch.full((128, 64), float("nan"), device=DEV)
-    assert lib.tt_atom_gemm(0, a.bfloat16().to(DEV).data_ptr(), b.bfloat16().to(DEV).data_ptr(), c.data_ptr()) == 0
-    ok, r, m = N.check_close(c, ref)
-    assert ok and m < 1e-4, (r, m)
-    ch = torch.full((128, 64), float("nan"), device=DEV, dtype=torch.float16)
-    assert lib.tt_atom_gemm(1, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), ch.data_ptr()) == 0
+    for blk in (0, 1, 6, 15):
+        a = torch.zeros(128, 256)
+        b = torch.randint(-3, 4, (64, 256), generator=g).float()
+        a[:, 16 * blk:16 * blk + 16] = torch.randint(-3, 4, (128, 16), generator=g).float()
+        a, b = a.half(), b.half()
+        assert lib.tt_readme_gemm(a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.data_ptr()) == 0
+        assert torch.equal(c.cpu(), N.gemm_ref(a, b)), blk
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 8, 9, 10])
+def test_other_mma_atoms(lib, variant):
+    # A [128, 192], B [192, 64]: bf16 / fp16 operands, fp32 / fp16 accumulators, row- and
+    # column-major accumulator tiles, even and odd base-tile counts per chunk (16x16x32 pairs and a
+    # 16x16x16 tail), square (0-4) and wide (8-10) operand tiles; integer data, so exact
+    bf16 = variant in (0, 4, 8)
+    half_acc = variant in (1, 9)
+    g = torch.Generator().manual_seed(30 + variant)
+    dt = torch.bfloat16 if bf16 else torch.float16
+    a = torch.randint(-3, 4, (128, 192), generator=g).to(dt)
+    b = torch.randint(-3, 4, (64, 192), generator=g).to(dt)
+    c = torch.full((128, 64), float("nan"), device=DEV, dtype=torch.float16 if half_acc else torch.float32)
+    assert lib.tt_atom_gemm(variant, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.data_ptr()) == 0
+    assert torch.equal(c.float().cpu(), N.gemm_ref(a, b))   # |C| <= 9 * 192 < 2048: exact in fp16 too
+    # random data against the fp32 oracle
+    a, b = oracle.make_c1_gemm_inputs(128, 64, 192, seed=40 + variant)
+    a, b = a.to(dt), b.to(dt)
+    assert lib.tt_atom_gemm(variant, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.data_ptr()) == 0
     ref = N.gemm_ref(a, b)
-    # 8 roundings to fp16 along K = 256 (one per 32-deep atom): a few fp16 ulps of |C| ~ 10
-    assert N.rel_l2(ch, ref) <= 2e-3 and N.max_abs(ch, ref) <= 5e-2, (N.rel_l2(ch, ref), N.max_abs(ch, ref))
+    if half_acc:
+        # the accumulator tile is rounded to fp16 once per gemm() call: a few fp16 ulps of |C| ~ 10
+        assert N.rel_l2(c, ref) <= 2e-3 and N.max_abs(c, ref) <= 5e-2, (N.rel_l2(c, ref), N.max_abs(c, ref))
+    else:
+        ok, r, m = N.check_close(c, ref)
+        assert ok and m < 1e-4, (r, m)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_single_mma_atom_on_one_base_tile(lib, variant):
+    # tests/cpp/cell/test_single_wmma.cu:222-231: one 16 x 16 x 16 atom against the naive loop
+    dt = torch.float16 if variant == 0 else torch.bfloat16
+    g = torch.Generator().manual_seed(50 + variant)
+    a = torch.randint(-4, 5, (16, 16), generator=g).to(dt)
+    b = torch.randint(-4, 5, (16, 16), generator=g).to(dt)   # [n, k] buffer = column-major k x n
+    c = torch.full((16, 16), float("nan"), device=DEV)
+    assert lib.tt_single_atom(variant, a.to(DEV).data_ptr(), b.to(DEV).data_ptr(), c.data_ptr()) == 0
+    assert torch.equal(c.cpu(), N.gemm_ref(a, b))
 
 
 @pytest.mark.parametrize("variant", range(6))
@@ -172,7 +215,7 @@ def test_ke_fused_two_gemms_composed_from_primitives(lib, variant):
         assert ok, (variant, i, r, ab)
 
 
-@pytest.mark.parametrize("variant", range(6))
+@pytest.mark.parametrize("variant", range(7))
 def test_ke_flash_attention_composed_from_primitives(lib, variant):
     # variants 0 and 1 are the reference's own cases (tests/python/test_flash_attn.py:
     # (64,128,128,128) plain, (128,128,128,128) causal; tiles (64,128,128,128))
@@ -241,14 +284,15 @@ def test_loader_fills_a_strided_subtile_through_registers(lib):
 
 # ---- warp helpers ------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("layout", range(3))
+@pytest.mark.parametrize("layout", range(4))
 @pytest.mark.parametrize("mode", range(3))
 def test_warp_offset_helpers_and_exec_counter(lib, layout, mode):
-    # (wavefront grid, its order, tile layout, base tile) of tt_warp_helpers' three layouts
+    # (wavefront grid, its order, tile layout, base tile) of tt_warp_helpers' four layouts
     wr, wc, wkind, tile, base = [
         (2, 2, L.ROW_MAJOR, L.row_major(128, 256, 512), (16, 32)),
         (4, 1, L.ROW_MAJOR, L.row_major(128, 64), (16, 32)),
         (2, 2, L.COL_MAJOR, L.col_major(128, 64, 256), (32, 16)),
+        (2, 2, L.ROW_MAJOR, L.row_major(128, 256, 512), (16, 16)),
     ][layout]
     name = ["kCont", "kRowReuseCont", "kColReuseCont"][mode]
     out = torch.full((wr * wc, 6), -1, dtype=torch.int64, device=DEV)

@@ -192,3 +192,26 @@ def test_golden_fixture():
             assert lay(i, j) == off
     for x, y, want in g["swizzle_3_3_3_points"]:
         assert L.swizzle(x * 64 + y, 3, 3, 3) == want
+
+
+def test_base_tile_lane_maps_cover_their_blocks():
+    # every element of the 16 x 16 (wide: 16 x 32 / 32 x 16) block is held by exactly one
+    # (lane, element) pair, for both orientations
+    for row_major in (True, False):
+        for per_lane in (4, 8):
+            rows, cols = L.base_tile_shape(row_major, per_lane)
+            seen = {L.base_tile_coord(lane, e, row_major, per_lane) for lane in range(64) for e in range(per_lane)}
+            assert seen == {(r, c) for r in range(rows) for c in range(cols)}
+    # the square row-major tile is the transpose of the square column-major one, lane for lane
+    for lane in range(64):
+        for e in range(4):
+            r, c = L.base_tile_coord(lane, e, True)
+            assert L.base_tile_coord(lane, e, False) == (c, r)
+
+
+def test_paired_square_tiles_feed_one_32_deep_instruction_consistently():
+    # two square base tiles adjacent in k, concatenated per lane, must give every k of the 32 to
+    # exactly one (lane group, element) slot, and A and B (same map) meet on equal k
+    for row in range(16):
+        ks = sorted(L.paired_k_assignment(row + 16 * g, e) for g in range(4) for e in range(8))
+        assert ks == list(range(32))

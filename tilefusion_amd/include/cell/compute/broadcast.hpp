@@ -1,7 +1,8 @@
-// Broadcast of a reduced vector (or a scalar) over an accumulator register tile (counterpart
-// of include/cell/compute/broadcast.hpp:14-187).  Row-major: src is the kRows x 4 vector that
-// SumReduce / MaxReduce produce and element (i, r) meets all columns of tile row
-// 16*i + 4*(l/16) + r.  The fused forms compute dst = f(dst, src) in place.
+// Broadcast of a reduced vector (or a scalar) over a register tile (counterpart of
+// include/cell/compute/broadcast.hpp:14-187).  Row-major: src is the vector SumReduce /
+// MaxReduce produce - one value per base-tile row, in column 0 - and element (i, 0) meets all
+// the lane's elements of tile row 16*i + l%16.  The fused forms compute dst = f(dst, src) in
+// place.
 #pragma once
 
 #include "cell/compute/math_functor.hpp"
@@ -13,6 +14,8 @@ namespace tl = tile_layout;
 template <typename SrcTile, typename DstTile, tl::Layout kLayout>
 struct Broadcast {
   using DType = typename DstTile::DType::DType;
+  static_assert(BaseTileTraits<typename DstTile::DType>::kIsRowMajor == (kLayout == tl::Layout::kRowMajor),
+                "a row vector is broadcast over row-major base tiles, a column vector over column-major ones");
   static constexpr int kRows = DstTile::kRows, kCols = DstTile::kCols;
   DEVICE void operator()(const SrcTile& src, DstTile& dst) {
 #pragma unroll
@@ -20,11 +23,11 @@ struct Broadcast {
 #pragma unroll
       for (int j = 0; j < kCols; ++j)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int e = 0; e < DstTile::DType::kNumel; ++e) {
           if constexpr (kLayout == tl::Layout::kRowMajor) {
-            dst(i, j)(r, 0) = src(i, r);
+            dst(i, j).mutable_data()[e] = src(i, 0);
           } else {
-            dst(i, j)(0, r) = src(r, j);
+            dst(i, j).mutable_data()[e] = src(0, j);
           }
         }
   }
@@ -33,6 +36,8 @@ struct Broadcast {
 template <typename SrcTile, typename DstTile, typename Functor, tl::Layout kLayout>
 struct BroadcastFuse {
   using DType = typename DstTile::DType::DType;
+  static_assert(BaseTileTraits<typename DstTile::DType>::kIsRowMajor == (kLayout == tl::Layout::kRowMajor),
+                "a row vector is broadcast over row-major base tiles, a column vector over column-major ones");
   static constexpr int kRows = DstTile::kRows, kCols = DstTile::kCols;
   DEVICE void operator()(const SrcTile& src, DstTile& dst) {
     Functor f;
@@ -41,11 +46,12 @@ struct BroadcastFuse {
 #pragma unroll
       for (int j = 0; j < kCols; ++j)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
+        for (int e = 0; e < DstTile::DType::kNumel; ++e) {
+          auto& d = dst(i, j).mutable_data()[e];
           if constexpr (kLayout == tl::Layout::kRowMajor) {
-            f(dst(i, j)(r, 0), src(i, r), dst(i, j)(r, 0));
+            f(d, src(i, 0), d);
           } else {
-            f(dst(i, j)(0, r), src(r, j), dst(i, j)(0, r));
+            f(d, src(0, j), d);
           }
         }
   }

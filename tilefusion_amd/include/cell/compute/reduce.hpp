@@ -1,15 +1,17 @@
-// Row / column reductions of accumulator register tiles (counterpart of
-// include/cell/compute/reduce.hpp:16-152) for the MFMA accumulator layout.
+// Row / column reductions of register tiles (counterpart of include/cell/compute/reduce.hpp:16-152).
 //
-// Row-major accumulator base tile: lane l holds column l%16 and rows 4*(l/16) .. +3, so the 16
-// lanes that share a row are exactly one DPP row of the wavefront.  Reducing along a row is
-//   1. fold the base tiles of a tile row inside the lane,
-//   2. one 4-step rotate-and-combine over the DPP row (no LDS crossbar traffic),
-// after which every lane of the DPP row holds the result.  The result vector of a tile with
-// kRows base-tile rows is RegTile<T, RowMajor<kRows, 4>>: element (i, r) belongs to tile row
-// 16*i + 4*(l/16) + r.  (On the reference's mma.m16n8k16 layout the vector is kRows x 2.)
-// The column-major form reduces column-major accumulator tiles along columns symmetrically
-// into RegTile<T, ColMajor<4, kCols>>.
+// A row-major base tile gives lane l the columns 4*(l/16) .. +3 of row l%16, so reducing
+// along rows is
+//   1. fold the lane's 4 elements of every base tile of a tile row,
+//   2. combine over the four lanes l%16 + {0, 16, 32, 48} that share the row (two register
+//      half-swaps, no LDS traffic), after which each of them holds the result.
+// A lane therefore owns ONE row per base-tile row: the natural result vector of a tile with
+// kRows base-tile rows is RegTile<T, RowMajor<kRows, 1>>, element (i, 0) belonging to tile row
+// 16*i + l%16.  Kernels written for the reference declare the vector as RowMajor<kRows, 2>
+// (its lanes own a top and a bottom row, include/cell/compute/reduce.hpp:52-68); any number of
+// columns is accepted and every column receives the same value, which the element-wise vector
+// ops and the Broadcast functors (they read column 0) are indifferent to.
+// Column-major base tiles reduce along columns symmetrically into ColMajor<n, kCols>.
 #pragma once
 
 #include "cell/compute/math_functor.hpp"
@@ -28,22 +30,23 @@ template <typename RegTile>
 struct Reduce<RegTile, tl::Layout::kRowMajor> {
   using BaseTile = typename RegTile::DType;
   using DType = typename BaseTile::DType;
-  static_assert(BaseTile::kNumel == 4 && BaseTile::kType == tl::Layout::kRowMajor,
-                "row reduction works on row-major accumulator base tiles");
+  static_assert(BaseTileTraits<BaseTile>::kIsRowMajor, "row reduction works on row-major base tiles");
   static constexpr int kRows = RegTile::kRows, kCols = RegTile::kCols;
 
   template <typename DstTile, typename Op>
   DEVICE void operator()(const RegTile& src, DstTile& dst, Op op) {
-    static_assert(DstTile::kRows == kRows && DstTile::kCols == 4, "the result vector is kRows x 4");
+    static_assert(DstTile::kRows == kRows && DstTile::kCols >= 1, "the result vector has one row per base-tile row");
 #pragma unroll
-    for (int i = 0; i < kRows; ++i)
+    for (int i = 0; i < kRows; ++i) {
+      float v = to_float(src(i, 0).data()[0]);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = to_float(src(i, 0)(r, 0));
+      for (int j = 0; j < kCols; ++j)
 #pragma unroll
-        for (int j = 1; j < kCols; ++j) v = op(v, to_float(src(i, j)(r, 0)));
-        dst(i, r) = from_float<DType>(row16_allreduce(v, op));
-      }
+        for (int e = (j == 0 ? 1 : 0); e < BaseTile::kNumel; ++e) v = op(v, to_float(src(i, j).data()[e]));
+      const auto out = from_float<typename DstTile::DType>(quad16_allreduce(v, op));
+#pragma unroll
+      for (int c = 0; c < DstTile::kCols; ++c) dst(i, c) = out;
+    }
   }
 };
 
@@ -51,22 +54,23 @@ template <typename RegTile>
 struct Reduce<RegTile, tl::Layout::kColMajor> {
   using BaseTile = typename RegTile::DType;
   using DType = typename BaseTile::DType;
-  static_assert(BaseTile::kNumel == 4 && BaseTile::kType == tl::Layout::kColMajor,
-                "column reduction works on column-major accumulator base tiles");
+  static_assert(!BaseTileTraits<BaseTile>::kIsRowMajor, "column reduction works on column-major base tiles");
   static constexpr int kRows = RegTile::kRows, kCols = RegTile::kCols;
 
   template <typename DstTile, typename Op>
   DEVICE void operator()(const RegTile& src, DstTile& dst, Op op) {
-    static_assert(DstTile::kRows == 4 && DstTile::kCols == kCols, "the result vector is 4 x kCols");
+    static_assert(DstTile::kCols == kCols && DstTile::kRows >= 1, "the result vector has one column per base-tile column");
 #pragma unroll
-    for (int j = 0; j < kCols; ++j)
+    for (int j = 0; j < kCols; ++j) {
+      float v = to_float(src(0, j).data()[0]);
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = to_float(src(0, j)(0, r));
+      for (int i = 0; i < kRows; ++i)
 #pragma unroll
-        for (int i = 1; i < kRows; ++i) v = op(v, to_float(src(i, j)(0, r)));
-        dst(r, j) = from_float<DType>(row16_allreduce(v, op));
-      }
+        for (int e = (i == 0 ? 1 : 0); e < BaseTile::kNumel; ++e) v = op(v, to_float(src(i, j).data()[e]));
+      const auto out = from_float<typename DstTile::DType>(quad16_allreduce(v, op));
+#pragma unroll
+      for (int r = 0; r < DstTile::kRows; ++r) dst(r, j) = out;
+    }
   }
 };
 

@@ -1,14 +1,10 @@
 // Global <-> register tile movers (counterpart of include/cell/copy/global_to_register.hpp:217-270)
-// in MFMA fragment order.
+// in the lane order of the base tiles (types/register.hpp).
 //
-// For every base tile of the RegTile a lane moves
-//   * operand, row-major global:    one 16-byte vector  - row l%16, columns 8*(l/16) .. +7 of the
-//                                   16 x 32 block;
-//   * operand, column-major global: one 16-byte vector  - column l%16, rows 8*(l/16) .. +7 of the
-//                                   32 x 16 block;
-//   * accumulator, row-major:       4 scalars           - column l%16, rows 4*(l/16) .. +3 of the
-//                                   16 x 16 block;
-//   * accumulator, column-major:    4 scalars           - row l%16, columns 4*(l/16) .. +3.
+// For every base tile of the RegTile a lane moves its 4 (wide tiles: 8) elements of row or
+// column l%16 of the block: as one 8- or 16-byte vector when the memory layout runs the same
+// way as the base tile (row-major tile from row-major memory, column-major from column-major),
+// element by element otherwise.
 // The WarpReuse mode is honoured as documented (include/cell/copy/constants.hpp:7-14): with
 // kRowReuseCont the wavefronts of a row share the row block and each reads ALL its columns.
 #pragma once
@@ -23,31 +19,8 @@ namespace tl = tile_layout;
 
 namespace detail {
 
-// element coordinates (row, col) inside a base tile's block and the contiguity of a lane's
-// elements, for lane `lane` and per-lane element index e
 template <typename BaseTile>
-struct FragmentMap {
-  using Traits = BaseTileTraits<BaseTile>;
-  DEVICE static void coord(int lane, int e, int& r, int& c) {
-    if constexpr (Traits::kIsOperand) {
-      if constexpr (Traits::kIsRowMajor) {
-        r = lane % 16;
-        c = 8 * (lane / 16) + e;
-      } else {
-        r = 8 * (lane / 16) + e;
-        c = lane % 16;
-      }
-    } else {
-      if constexpr (Traits::kIsRowMajor) {
-        r = 4 * (lane / 16) + e;
-        c = lane % 16;
-      } else {
-        r = lane % 16;
-        c = 4 * (lane / 16) + e;
-      }
-    }
-  }
-};
+using FragmentMap = BaseTileTraits<BaseTile>;
 
 // extent of the block one base tile covers in memory, in the form warp::ExecCounter takes
 template <typename BaseTile>
@@ -55,6 +28,30 @@ struct BaseExtent {
   static constexpr int kRows = BaseTileTraits<BaseTile>::kRows;
   static constexpr int kCols = BaseTileTraits<BaseTile>::kCols;
 };
+
+// a lane's elements of one base tile as one vector
+template <int kBytes>
+struct VecOfBytes;
+template <>
+struct VecOfBytes<8> {
+  using type = uint2;
+};
+template <>
+struct VecOfBytes<16> {
+  using type = uint4;
+};
+template <>
+struct VecOfBytes<32> {
+  struct type {
+    uint4 lo, hi;
+  };
+};
+
+// the lane's elements are contiguous in a tile with these strides
+template <typename BaseTile, typename Tile>
+inline constexpr bool kLaneContiguous =
+    (BaseTileTraits<BaseTile>::kIsRowMajor && Tile::kColStride == 1) ||
+    (!BaseTileTraits<BaseTile>::kIsRowMajor && Tile::kRowStride == 1);
 
 // The register tile must be exactly the base tiles a wavefront walks over in its share.
 template <typename Tile, typename Reg, typename WarpLayout, WarpReuse kMode>
@@ -89,11 +86,10 @@ struct GlobalToRegLoader {
         detail::FragmentMap<BaseTile>::coord(lane, 0, r, c);
         r += i * Traits::kRows;
         c += j * Traits::kCols;
-        constexpr bool kContig = Traits::kIsOperand && ((Traits::kIsRowMajor && Global::kColStride == 1) ||
-                                                        (!Traits::kIsRowMajor && Global::kRowStride == 1));
-        if constexpr (kContig) {
-          *reinterpret_cast<uint4*>(out) =
-              *reinterpret_cast<const uint4*>(base + ptrdiff_t(r) * Global::kRowStride + ptrdiff_t(c) * Global::kColStride);
+        if constexpr (detail::kLaneContiguous<BaseTile, Global>) {
+          using Vec = typename detail::VecOfBytes<sizeof(BaseTile)>::type;
+          *reinterpret_cast<Vec*>(out) =
+              *reinterpret_cast<const Vec*>(base + ptrdiff_t(r) * Global::kRowStride + ptrdiff_t(c) * Global::kColStride);
         } else {
 #pragma unroll
           for (int e = 0; e < BaseTile::kNumel; ++e) {
@@ -127,13 +123,23 @@ struct RegToGlobalStorer {
 #pragma unroll
       for (int j = 0; j < Reg::kCols; ++j) {
         const DType* in = src(i, j).data();
+        if constexpr (detail::kLaneContiguous<BaseTile, Global>) {
+          using Vec = typename detail::VecOfBytes<sizeof(BaseTile)>::type;
+          int r, c;
+          detail::FragmentMap<BaseTile>::coord(lane, 0, r, c);
+          r += i * Traits::kRows;
+          c += j * Traits::kCols;
+          *reinterpret_cast<Vec*>(base + ptrdiff_t(r) * Global::kRowStride + ptrdiff_t(c) * Global::kColStride) =
+              *reinterpret_cast<const Vec*>(in);
+        } else {
 #pragma unroll
-        for (int e = 0; e < BaseTile::kNumel; ++e) {
-          int rr, cc;
-          detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
-          rr += i * Traits::kRows;
-          cc += j * Traits::kCols;
-          base[ptrdiff_t(rr) * Global::kRowStride + ptrdiff_t(cc) * Global::kColStride] = in[e];
+          for (int e = 0; e < BaseTile::kNumel; ++e) {
+            int rr, cc;
+            detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
+            rr += i * Traits::kRows;
+            cc += j * Traits::kCols;
+            base[ptrdiff_t(rr) * Global::kRowStride + ptrdiff_t(cc) * Global::kColStride] = in[e];
+          }
         }
       }
   }

@@ -1,6 +1,8 @@
-// LDS <-> register tile movers in MFMA fragment order (counterpart of
-// include/cell/copy/shared_to_register.hpp:248-367; there is no ldmatrix on CDNA - an operand
-// fragment is simply one ds_read_b128 per lane because both MFMA operands are contiguous in k).
+// LDS <-> register tile movers in the lane order of the base tiles (counterpart of
+// include/cell/copy/shared_to_register.hpp:248-367; there is no ldmatrix on CDNA - a lane's part
+// of a base tile is one ds_read_b64 (wide tiles: ds_read_b128) when the LDS layout runs the same
+// way as the base tile, because both MFMA operands are contiguous in k).  The swizzle moves
+// whole 16-byte vectors, so a lane's 8 or 16 aligned bytes stay together.
 #pragma once
 
 #include "cell/copy/global_to_register.hpp"
@@ -31,14 +33,13 @@ struct SharedToRegLoader {
 #pragma unroll
       for (int j = 0; j < Reg::kCols; ++j) {
         DType* out = dst(i, j).mutable_data();
-        constexpr bool kContig = Traits::kIsOperand && ((Traits::kIsRowMajor && Shared::kColStride == 1) ||
-                                                        (!Traits::kIsRowMajor && Shared::kRowStride == 1));
-        if constexpr (kContig) {
+        if constexpr (detail::kLaneContiguous<BaseTile, Shared> && sizeof(BaseTile) <= 16) {
+          using Vec = typename detail::VecOfBytes<sizeof(BaseTile)>::type;
           int r, c;
           detail::FragmentMap<BaseTile>::coord(lane, 0, r, c);
           r += i * Traits::kRows;
           c += j * Traits::kCols;
-          *reinterpret_cast<uint4*>(out) = *reinterpret_cast<const uint4*>(
+          *reinterpret_cast<Vec*>(out) = *reinterpret_cast<const Vec*>(
               base + src.fetch_physical_offset(warp_off + r * Shared::kRowStride + c * Shared::kColStride));
         } else {
 #pragma unroll
@@ -74,13 +75,24 @@ struct RegToSharedStorer {
 #pragma unroll
       for (int j = 0; j < Reg::kCols; ++j) {
         const DType* in = src(i, j).data();
+        if constexpr (detail::kLaneContiguous<BaseTile, Shared> && sizeof(BaseTile) <= 16) {
+          using Vec = typename detail::VecOfBytes<sizeof(BaseTile)>::type;
+          int r, c;
+          detail::FragmentMap<BaseTile>::coord(lane, 0, r, c);
+          r += i * Traits::kRows;
+          c += j * Traits::kCols;
+          *reinterpret_cast<Vec*>(
+              base + dst.fetch_physical_offset(warp_off + r * Shared::kRowStride + c * Shared::kColStride)) =
+              *reinterpret_cast<const Vec*>(in);
+        } else {
 #pragma unroll
-        for (int e = 0; e < BaseTile::kNumel; ++e) {
-          int rr, cc;
-          detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
-          rr += i * Traits::kRows;
-          cc += j * Traits::kCols;
-          base[dst.fetch_physical_offset(warp_off + rr * Shared::kRowStride + cc * Shared::kColStride)] = in[e];
+          for (int e = 0; e < BaseTile::kNumel; ++e) {
+            int rr, cc;
+            detail::FragmentMap<BaseTile>::coord(lane, e, rr, cc);
+            rr += i * Traits::kRows;
+            cc += j * Traits::kCols;
+            base[dst.fetch_physical_offset(warp_off + rr * Shared::kRowStride + cc * Shared::kColStride)] = in[e];
+          }
         }
       }
   }

@@ -35,4 +35,18 @@ DEVICE float row16_allreduce(float x, Op op) {
   return x;
 }
 
+// Combine a value over the four lanes l%16, l%16 + 16, l%16 + 32, l%16 + 48 (the lanes that
+// share a row of a row-major base tile, or a column of a column-major one); every lane
+// receives the result.  v_permlane16_swap / v_permlane32_swap exchange 16- and 32-lane halves
+// between two registers in one instruction, without the LDS crossbar.
+template <typename Op>
+DEVICE float quad16_allreduce(float x, Op op) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  auto s16 = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  x = op(__builtin_bit_cast(float, (unsigned)s16[0]), __builtin_bit_cast(float, (unsigned)s16[1]));
+  const unsigned v = __builtin_bit_cast(unsigned, x);
+  auto s32 = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return op(__builtin_bit_cast(float, (unsigned)s32[0]), __builtin_bit_cast(float, (unsigned)s32[1]));
+}
+
 }  // namespace tilefusion::cell

@@ -6,9 +6,10 @@
 // Differences from the reference: running max / sum are fp32 and start at -inf / 0 (the
 // reference keeps them in fp16 and starts the max at 0); the output stays un-normalised until
 // the end (one divide instead of one per key tile); the causal mask skips key tiles that lie
-// entirely above the diagonal.  exp(S - max) is rounded to fp16 and re-laid-out through an LDS
-// tile for the second MFMA.  (The library's tuned entry point tf_flash_attention_fwd_f16
-// computes the scores transposed instead and needs no re-layout.)
+// entirely above the diagonal.  The score tile is a tile of row-major base tiles, which is the
+// layout of an A operand (types/register.hpp): exp(S - max) is rounded to fp16 element by element
+// and fed to the second gemm() straight from registers, as in the reference.  Q and K are held as
+// wide 16 x 32 base tiles when kTK is a multiple of 32.
 //
 // When one k-chunk covers the whole head dimension (kTK == kK) the Q tile is fetched once and
 // stays in registers (the reference reloads it per key tile,
@@ -48,49 +49,60 @@ struct FlashAttentionTraits {
   static constexpr int kTN = dim_size<1, CtaTileShape>;
   static constexpr int kTK = dim_size<2, CtaTileShape>;
   static constexpr int kTP = dim_size<3, CtaTileShape>;
-  static_assert(kTK % 32 == 0 && kTN % 32 == 0 && kTP % 16 == 0 && (kTM / kWarpPerRow) % 16 == 0,
-                "tile sizes must be whole MFMA base tiles");
+  static_assert(kTK % 16 == 0 && kTN % 16 == 0 && kTP % 16 == 0 && (kTM / kWarpPerRow) % 16 == 0,
+                "tile sizes must be whole base tiles");
   static constexpr double kSoftmaxScale = kSoftmaxScale_;
   static constexpr bool kIsCausal = kIsCausal_;
-  static constexpr int kRowsPerWarp = kTM / kWarpPerRow;
+  static constexpr bool kWideOperands = kTK % 32 == 0;
+  static constexpr int kOperandK = kWideOperands ? 32 : BaseShape::kCols;
+  template <typename T>
+  using OperandRowMajor = std::conditional_t<kWideOperands, RegTile<T, tl::RowMajor<1, 8>>, BaseTileRowMajor<T>>;
+  template <typename T>
+  using OperandColMajor = std::conditional_t<kWideOperands, RegTile<T, tl::ColMajor<8, 1>>, BaseTileColMajor<T>>;
 
   using GlobalQ = GlobalTile<InType, tl::RowMajor<kTM, kK>>;
   using GIteratorQ = GTileIterator<GlobalQ, TileShape<kTM, kTK>>;
   using SharedQ = SharedTile<InType, tl::RowMajor<kTM, kTK>, true, kSharedAccess>;
-  using RegQ = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kRowsPerWarp / 16, kTK / 32>>;
+  static constexpr int kQMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kQKs = kTK / kOperandK;
+  using RegQ = RegTile<OperandRowMajor<InType>, tl::RowMajor<kQMs, kQKs>>;
   using SharedQLoader = GlobalToSharedLoader<SharedQ, WarpLayout>;
   using RegQLoader = SharedToRegLoader<RegQ, WarpLayout, WarpReuse::kRowReuseCont>;
 
   using GlobalK = GlobalTile<InType, tl::ColMajor<kK, kN>>;
   using GIteratorK = GTileIterator<GlobalK, TileShape<kTK, kTN>>;
   using SharedK = SharedTile<InType, tl::ColMajor<kTK, kTN>, true, kSharedAccess>;
-  using RegK = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kTN / 16>>;
+  static constexpr int kKKs = kTK / kOperandK;
+  static constexpr int kKNs = kTN / kWarpPerCol / BaseShape::kCols;
+  using RegK = RegTile<OperandColMajor<InType>, tl::ColMajor<kKKs, kKNs>>;
   using SharedKLoader = GlobalToSharedLoader<SharedK, WarpLayout>;
   using RegKLoader = SharedToRegLoader<RegK, WarpLayout, WarpReuse::kColReuseCont>;
 
   using GlobalV = GlobalTile<InType, tl::ColMajor<kN, kTP>>;
   using GIteratorV = GTileIterator<GlobalV, TileShape<kTN, kTP>>;
   using SharedV = SharedTile<InType, tl::ColMajor<kTN, kTP>, true, kSharedAccess>;
-  using RegV = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTN / 32, kTP / 16>>;
+  static constexpr int kVNs = kTN / BaseShape::kRows;
+  static constexpr int kVPs = kTP / kWarpPerCol / BaseShape::kCols;
+  using RegV = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kVNs, kVPs>>;
   using SharedVLoader = GlobalToSharedLoader<SharedV, WarpLayout>;
   using RegVLoader = SharedToRegLoader<RegV, WarpLayout, WarpReuse::kColReuseCont>;
 
   using GlobalO = GlobalTile<OutType, tl::RowMajor<kTM, kTP, kP>>;
-  using RegO = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kRowsPerWarp / 16, kTP / 16>>;
-  using RegOCast = RegTile<BaseTileAccRowMajor<OutType>, tl::RowMajor<kRowsPerWarp / 16, kTP / 16>>;
+  static constexpr int kOMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kOPs = kTP / kWarpPerCol / BaseShape::kCols;
+  using RegO = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kOMs, kOPs>>;
+  using RegOCast = RegTile<BaseTileRowMajor<OutType>, tl::RowMajor<kOMs, kOPs>>;
   using ConvertO = compute::RegTileConvert<RegO, RegOCast>;
   using OStorer = RegToGlobalStorer<GlobalO, RegOCast, WarpLayout>;
 
-  using RegAcc = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kRowsPerWarp / 16, kTN / 16>>;
-  using RegAccCast = RegTile<BaseTileAccRowMajor<InType>, tl::RowMajor<kRowsPerWarp / 16, kTN / 16>>;
+  static constexpr int kAccMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kAccNs = kTN / kWarpPerCol / BaseShape::kCols;
+  using RegAcc = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kAccMs, kAccNs>>;
+  using RegAccCast = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAccMs, kAccNs>>;
   using ConvertAcc = compute::RegTileConvert<RegAcc, RegAccCast>;
-  using SharedP = SharedTile<InType, tl::RowMajor<kTM, kTN>, true, kSharedAccess>;
-  using RegP = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kRowsPerWarp / 16, kTN / 32>>;
-  using StorerP = RegToSharedStorer<RegAccCast, WarpLayout>;
-  using LoaderP = SharedToRegLoader<RegP, WarpLayout, WarpReuse::kRowReuseCont>;
 
-  // one statistic per row a lane owns: 4 per base-tile row (fp32)
-  using RegVec = RegTile<AccType, tl::RowMajor<kRowsPerWarp / 16, 4>>;
+  // one statistic per row a lane owns: one per base-tile row (fp32)
+  using RegVec = RegTile<AccType, tl::RowMajor<kAccMs, 1>>;
   using RowMax = compute::MaxReduce<RegAcc, tl::Layout::kRowMajor>;
   using RowSum = compute::SumReduce<RegAcc, tl::Layout::kRowMajor>;
   using BroadcastSub = compute::BroadcastSub<RegVec, RegAcc, tl::Layout::kRowMajor>;
@@ -107,8 +119,7 @@ struct FlashAttentionTraits {
 
   // the whole head dimension in one chunk: Q is fetched once (see above)
   static constexpr bool kWholeK = kTK == kK;
-  static constexpr int kSharedBytes =
-      (SharedQ::kNumel + SharedK::kNumel + SharedV::kNumel + SharedP::kNumel) * (int)sizeof(InType);
+  static constexpr int kSharedBytes = (SharedQ::kNumel + SharedK::kNumel + SharedV::kNumel) * (int)sizeof(InType);
 };
 
 template <typename InType, typename AccType, typename OutType, typename KeTraits>
@@ -126,7 +137,6 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
   typename T::SharedQ sQ(lds);
   typename T::SharedK sK(lds + T::SharedQ::kNumel);
   typename T::SharedV sV(lds + T::SharedQ::kNumel + T::SharedK::kNumel);
-  typename T::SharedP sP(lds + T::SharedQ::kNumel + T::SharedK::kNumel + T::SharedV::kNumel);
 
   typename T::GIteratorQ gQs(Q);
   typename T::GIteratorK gKs(K);
@@ -140,7 +150,6 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
   typename T::RegQ rQ;
   typename T::RegK rK;
   typename T::RegV rV;
-  typename T::RegP rP;
   typename T::RegAcc s;
   typename T::RegAccCast p_half;
   typename T::RegO o;
@@ -152,7 +161,7 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
   // causal: key tiles that start after the last row of this workgroup contribute nothing
   const int n_tiles = T::kIsCausal ? min((int)T::GIteratorV::sc0, (row_base + kTM + kTN - 1) / kTN)
                                    : (int)T::GIteratorV::sc0;
-  // scale, mask, online softmax of the score tile `s` of key tile n; leaves the fp16 weights in sP
+  // scale, mask, online softmax of the score tile `s` of key tile n; leaves the fp16 weights in p_half
   auto softmax_tile = [&](int n) {
     typename T::ApplyScoreScale scale;
     scale(s, AccType(T::kSoftmaxScale), s);
@@ -188,8 +197,6 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
 
     typename T::ConvertAcc to_half;
     to_half(s, p_half);
-    typename T::StorerP store_p;
-    store_p(p_half, sP);
   };
 
   if constexpr (T::kWholeK) {
@@ -203,13 +210,10 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
       load_rk(sK, rK);
       compute::gemm(rQ, rK, s);
       softmax_tile(n);
-      __syncthreads();   // the weights are in LDS
-      typename T::LoaderP load_p;
-      load_p(sP, rP);
       load_rv(sV, rV);
-      compute::gemm(rP, rV, o);
+      compute::gemm(p_half, rV, o);
       s.clear();
-      __syncthreads();   // nobody still reads this tile or its weights
+      __syncthreads();   // nobody still reads this tile
     }
   } else {
     for (int n = 0; n < n_tiles; ++n) {
@@ -225,12 +229,8 @@ DEVICE void ke_flash_attention(const InType* dQ, const InType* dK, const InType*
         __syncthreads();
       }
       softmax_tile(n);
-      __copy_async();
-      __syncthreads();
-      typename T::LoaderP load_p;
-      load_p(sP, rP);
       load_rv(sV, rV);
-      compute::gemm(rP, rV, o);
+      compute::gemm(p_half, rV, o);
       s.clear();
       __syncthreads();
     }

@@ -3,11 +3,10 @@
 // D row-major and B, C column-major; one workgroup per [kTM, kTP] tile of D; the intermediate
 // A*B tile never leaves the chip.
 //
-// The first product arrives in the MFMA accumulator layout (a lane owns a column), the second
-// MFMA wants it in the row-major operand layout (a lane owns a row): the fp16-rounded tile is
-// re-laid-out through an LDS tile with RegToSharedStorer / SharedToRegLoader.  (The library's
-// tuned entry point tf_fused_two_gemms_f16 avoids that round trip by computing the first
-// product transposed.)
+// The accumulator tile of the first product is a tile of row-major base tiles - the layout of an
+// A operand (types/register.hpp) - so, as in the reference, it is converted to fp16 element by
+// element and fed to the second gemm() straight from registers.  The first product's own
+// operands are held as wide 16 x 32 base tiles when kTK is a multiple of 32.
 #pragma once
 
 #include "cell/mod.hpp"
@@ -24,7 +23,7 @@ struct FusedTwoGemmsTraits {
   using InType = InType_;
   using AccType = AccType_;
   using WarpLayout = WarpLayout_;
-  using BaseShape = BaseTileShape<InType>;
+  using BaseShape = BaseTileShape<InType>;  // 16 x 16
   static constexpr int kThreads = tl::get_numel<WarpLayout> * WARP_SIZE;
   static constexpr int kWarpPerRow = tl::num_rows<WarpLayout>;
   static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
@@ -32,48 +31,58 @@ struct FusedTwoGemmsTraits {
   static constexpr int kM = kM_, kN = kN_, kK = kK_, kP = kP_;
   static constexpr int kTM = kTM_, kTN = kTN_, kTK = kTK_, kTP = kTP_;
   static constexpr int kSharedAccess = 64;
-  static_assert(kTK % 32 == 0 && kTN % 32 == 0 && kTP % 16 == 0 && (kTM / kWarpPerRow) % 16 == 0,
-                "tile sizes must be whole MFMA base tiles");
+  static_assert(kTK % 16 == 0 && kTN % 16 == 0 && kTP % 16 == 0 && (kTM / kWarpPerRow) % 16 == 0,
+                "tile sizes must be whole base tiles");
+  static constexpr bool kWideOperands = kTK % 32 == 0;
+  static constexpr int kOperandK = kWideOperands ? 32 : BaseShape::kCols;
+  template <typename T>
+  using OperandRowMajor = std::conditional_t<kWideOperands, RegTile<T, tl::RowMajor<1, 8>>, BaseTileRowMajor<T>>;
+  template <typename T>
+  using OperandColMajor = std::conditional_t<kWideOperands, RegTile<T, tl::ColMajor<8, 1>>, BaseTileColMajor<T>>;
 
   using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK>>;
   using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
   using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, true, kSharedAccess>;
-  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kTM / kWarpPerRow / 16, kTK / 32>>;
+  static constexpr int kAMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kAKs = kTK / kOperandK;
+  using RegA = RegTile<OperandRowMajor<InType>, tl::RowMajor<kAMs, kAKs>>;
   using SharedALoader = GlobalToSharedLoader<SharedA, WarpLayout>;
   using RegALoader = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
 
   using GlobalB = GlobalTile<InType, tl::ColMajor<kK, kN>>;
   using GIteratorB = GTileIterator<GlobalB, TileShape<kTK, kTN>>;
   using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, true, kSharedAccess>;
-  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTK / 32, kTN / 16>>;
+  static constexpr int kBKs = kTK / kOperandK;
+  static constexpr int kBNs = kTN / kWarpPerCol / BaseShape::kCols;
+  using RegB = RegTile<OperandColMajor<InType>, tl::ColMajor<kBKs, kBNs>>;
   using SharedBLoader = GlobalToSharedLoader<SharedB, WarpLayout>;
   using RegBLoader = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
 
   using GlobalC = GlobalTile<InType, tl::ColMajor<kN, kTP>>;
   using GIteratorC = GTileIterator<GlobalC, TileShape<kTN, kTP>>;
   using SharedC = SharedTile<InType, tl::ColMajor<kTN, kTP>, true, kSharedAccess>;
-  using RegC = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kTN / 32, kTP / 16>>;
+  static constexpr int kCNs = kTN / BaseShape::kRows;
+  static constexpr int kCPs = kTP / kWarpPerCol / BaseShape::kCols;
+  using RegC = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kCNs, kCPs>>;
   using SharedCLoader = GlobalToSharedLoader<SharedC, WarpLayout>;
   using RegCLoader = SharedToRegLoader<RegC, WarpLayout, WarpReuse::kColReuseCont>;
 
-  // intermediate tile: fp32 accumulators -> fp16 in accumulator layout -> LDS -> operand layout
-  using RegAcc = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kTM / kWarpPerRow / 16, kTN / 16>>;
-  using RegAccCast = RegTile<BaseTileAccRowMajor<InType>, tl::RowMajor<kTM / kWarpPerRow / 16, kTN / 16>>;
+  // intermediate tile: fp32 accumulators, converted in place to the A operand of the second product
+  static constexpr int kAccMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kAccNs = kTN / kWarpPerCol / BaseShape::kCols;
+  using RegAcc = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kAccMs, kAccNs>>;
+  using RegAccCast = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAccMs, kAccNs>>;
   using ConvertHalf = compute::RegTileConvert<RegAcc, RegAccCast>;
-  using SharedP = SharedTile<InType, tl::RowMajor<kTM, kTN>, true, kSharedAccess>;
-  using RegP = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kTM / kWarpPerRow / 16, kTN / 32>>;
-  using StorerP = RegToSharedStorer<RegAccCast, WarpLayout>;
-  using LoaderP = SharedToRegLoader<RegP, WarpLayout, WarpReuse::kRowReuseCont>;
 
   using GlobalD = GlobalTile<InType, tl::RowMajor<kTM, kTP, kP>>;
-  using SharedD = SharedTile<InType, tl::RowMajor<kTM, kTP>, false>;
-  using RegD = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kTM / kWarpPerRow / 16, kTP / 16>>;
-  using RegDCast = RegTile<BaseTileAccRowMajor<InType>, tl::RowMajor<kTM / kWarpPerRow / 16, kTP / 16>>;
-  using ConvertD = compute::RegTileConvert<RegD, RegDCast>;
-  using StorerD = RegToGlobalStorer<GlobalD, RegDCast, WarpLayout>;
+  static constexpr int kDMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kDPs = kTP / kWarpPerCol / BaseShape::kCols;
+  using RegD = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kDMs, kDPs>>;
+  using RegDHalf = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kDMs, kDPs>>;
+  using ConvertD = compute::RegTileConvert<RegD, RegDHalf>;
+  using StorerD = RegToGlobalStorer<GlobalD, RegDHalf, WarpLayout>;
 
-  static constexpr int kSharedBytes =
-      (SharedA::kNumel + SharedB::kNumel + SharedC::kNumel + SharedP::kNumel) * (int)sizeof(InType);
+  static constexpr int kSharedBytes = (SharedA::kNumel + SharedB::kNumel + SharedC::kNumel) * (int)sizeof(InType);
 };
 
 template <typename InType, typename AccType, typename KeTraits>
@@ -90,7 +99,6 @@ DEVICE void ke_fused_two_gemms(const InType* dA, const InType* dB, const InType*
   typename T::SharedA sA(lds);
   typename T::SharedB sB(lds + T::SharedA::kNumel);
   typename T::SharedC sC(lds + T::SharedA::kNumel + T::SharedB::kNumel);
-  typename T::SharedP sP(lds + T::SharedA::kNumel + T::SharedB::kNumel + T::SharedC::kNumel);
 
   typename T::GIteratorA gAs(A);
   typename T::GIteratorB gBs(B);
@@ -104,7 +112,6 @@ DEVICE void ke_fused_two_gemms(const InType* dA, const InType* dB, const InType*
   typename T::RegA rA;
   typename T::RegB rB;
   typename T::RegC rC;
-  typename T::RegP rP;
   typename T::RegAcc acc;
   typename T::RegAccCast acc_half;
   typename T::RegD rD;
@@ -123,18 +130,12 @@ DEVICE void ke_fused_two_gemms(const InType* dA, const InType* dB, const InType*
     }
     typename T::ConvertHalf to_half;
     to_half(acc, acc_half);
-    typename T::StorerP store_p;
-    store_p(acc_half, sP);
-    __copy_async();
-    __syncthreads();
-    typename T::LoaderP load_p;
-    load_p(sP, rP);
     load_rc(sC, rC);
-    compute::gemm(rP, rC, rD);
+    compute::gemm(acc_half, rC, rD);
     acc.clear();
-    __syncthreads();  // sP / sC are overwritten by the next n-chunk
+    __syncthreads();  // sC is overwritten by the next n-chunk
   }
-  typename T::RegDCast out;
+  typename T::RegDHalf out;
   typename T::ConvertD to_out;
   to_out(rD, out);
   typename T::GlobalD gD(D);

@@ -7,9 +7,11 @@
 // parameter and any kernel written against the tile API composes the same way.  The library's
 // own tuned GEMM entry point (tf_gemm_f16) is a separate hand-scheduled kernel.
 //
-// Differences from the reference that follow from the hardware: a wavefront has 64 lanes
-// (kThreads = |WarpLayout| * 64) and the MFMA reduces 32 values of k per instruction (kRK is
-// rounded up to a multiple of 32).
+// The traits are the reference's, formula for formula (base tiles are 16 x 16, a register step
+// kRK is a multiple of 16); what follows from the hardware: a wavefront has 64 lanes
+// (kThreads = |WarpLayout| * 64), and when kRK is a multiple of 32 the operand fragments are
+// held as wide 16 x 32 base tiles (one 16-byte LDS read per lane and MFMA instead of two
+// 8-byte ones; same arithmetic).
 //
 // Three schedules, as in the reference:
 //   ke_gemm                  load chunk, wait, multiply (kNumStages >= 2: two LDS buffers, the
@@ -36,7 +38,7 @@ struct KeGemmTraits {
   using InType = InType_;
   using AccType = AccType_;
   using WarpLayout = WarpLayout_;
-  using BaseShape = BaseTileShape<InType>;  // 16 x 32 operand block
+  using BaseShape = BaseTileShape<InType>;  // 16 x 16
   static constexpr int kNumStages = kNumStages_;
 
   static constexpr int kThreads = tl::get_numel<WarpLayout> * WARP_SIZE;
@@ -44,18 +46,24 @@ struct KeGemmTraits {
   static constexpr int kWarpPerCol = tl::num_cols<WarpLayout>;
 
   static constexpr int kM = kM_, kN = kN_, kK = kK_;
-  static constexpr int kTM = kTM_, kTN = kTN_, kTK = kTK_;
-  static constexpr int kRK = kRK_ < BaseShape::kCols ? BaseShape::kCols : kRK_;
-  static_assert(kTK % kRK == 0 && kRK % BaseShape::kCols == 0, "kTK must be a multiple of kRK (a multiple of 32)");
+  static constexpr int kTM = kTM_, kTN = kTN_, kTK = kTK_, kRK = kRK_;
+  static_assert(kTK % kRK == 0 && kRK % BaseShape::kCols == 0, "kTK must be a multiple of kRK (a multiple of 16)");
   static constexpr bool kSwizzled = true;
+  // operand fragments as wide base tiles when a register step is whole 32-deep blocks
+  static constexpr bool kWideOperands = kRK % 32 == 0;
+  static constexpr int kOperandK = kWideOperands ? 32 : BaseShape::kCols;
+  template <typename T>
+  using OperandRowMajor = std::conditional_t<kWideOperands, RegTile<T, tl::RowMajor<1, 8>>, BaseTileRowMajor<T>>;
+  template <typename T>
+  using OperandColMajor = std::conditional_t<kWideOperands, RegTile<T, tl::ColMajor<8, 1>>, BaseTileColMajor<T>>;
 
   using GlobalA = GlobalTile<InType, tl::RowMajor<kTM, kK, kK>>;
   using GIteratorA = GTileIterator<GlobalA, TileShape<kTM, kTK>>;
   using SharedA = SharedTile<InType, tl::RowMajor<kTM, kTK>, kSwizzled, kSharedAccess>;
   using SIteratorA = STileIterator<SharedA, TileShape<kTM, kRK>>;
   static constexpr int kAMs = kTM / kWarpPerRow / BaseShape::kRows;
-  static constexpr int kAKs = kRK / BaseShape::kCols;
-  using RegA = RegTile<BaseTileRowMajor<InType>, tl::RowMajor<kAMs, kAKs>>;
+  static constexpr int kAKs = kRK / kOperandK;
+  using RegA = RegTile<OperandRowMajor<InType>, tl::RowMajor<kAMs, kAKs>>;
   using G2SLoaderA = GlobalToSharedLoader<SharedA, WarpLayout>;
   using S2RLoaderA = SharedToRegLoader<RegA, WarpLayout, WarpReuse::kRowReuseCont>;
 
@@ -64,17 +72,17 @@ struct KeGemmTraits {
   using SharedB = SharedTile<InType, tl::ColMajor<kTK, kTN>, kSwizzled, kSharedAccess>;
   using SIteratorB = STileIterator<SharedB, TileShape<kRK, kTN>>;
   static_assert(GIteratorA::sc1 == GIteratorB::sc0 && SIteratorA::sc1 == SIteratorB::sc0, "mismatched K dimension");
-  static constexpr int kBKs = kRK / BaseShape::kCols;                   // 32 values of k per base tile
-  static constexpr int kBNs = kTN / kWarpPerCol / BaseShape::kRows;     // 16 columns per base tile
-  using RegB = RegTile<BaseTileColMajor<InType>, tl::ColMajor<kBKs, kBNs>>;
+  static constexpr int kBKs = kRK / kOperandK;
+  static constexpr int kBNs = kTN / kWarpPerCol / BaseShape::kCols;
+  using RegB = RegTile<OperandColMajor<InType>, tl::ColMajor<kBKs, kBNs>>;
   using G2SLoaderB = GlobalToSharedLoader<SharedB, WarpLayout>;
   using S2RLoaderB = SharedToRegLoader<RegB, WarpLayout, WarpReuse::kColReuseCont>;
 
   using GlobalC = GlobalTile<AccType, tl::RowMajor<kTM, kTN, kN>>;
   using SharedC = SharedTile<AccType, tl::RowMajor<kTM, kTN>, false>;
-  static constexpr int kCMs = kTM / kWarpPerRow / 16;
-  static constexpr int kCNs = kTN / kWarpPerCol / 16;
-  using RegC = RegTile<BaseTileAccRowMajor<AccType>, tl::RowMajor<kCMs, kCNs>>;
+  static constexpr int kCMs = kTM / kWarpPerRow / BaseShape::kRows;
+  static constexpr int kCNs = kTN / kWarpPerCol / BaseShape::kCols;
+  using RegC = RegTile<BaseTileRowMajor<AccType>, tl::RowMajor<kCMs, kCNs>>;
   using RegAcc = RegTile<BaseTileRowMajor<float>, tl::RowMajor<kCMs, kCNs>>;
   using R2GStorerC = RegToGlobalStorer<GlobalC, RegC, WarpLayout>;
   using R2SStorerC = RegToSharedStorer<RegC, WarpLayout>;

@@ -1,10 +1,13 @@
 // Element types and the machine constants the tile types are sized by.
 //
-// Counterpart of include/types/base.hpp:20-68, re-derived for CDNA4: the matrix instruction the
-// tiles are built around is v_mfma_f32_16x16x32_{f16,bf16}.  A 16-bit OPERAND base tile is
-// therefore 16 x 32 (row-major A) or 32 x 16 (column-major B) with 8 contiguous-in-k elements
-// per lane, and an ACCUMULATOR base tile is 16 x 16 with 4 elements per lane - not the 16 x 16
-// / 8-per-thread tile of mma.m16n8k16 on a 32-lane warp.
+// Counterpart of include/types/base.hpp:20-68.  A base tile is the reference's square 16 x 16
+// block for every element type, so the tile-count arithmetic of kernels written against the
+// reference (kTM / kWarpPerRow / BaseShape::kRows, kRK / BaseShape::kCols, ...) carries over
+// unchanged; what differs is how the block is spread over the lanes: 64 lanes hold 4 elements
+// each (types/register.hpp) instead of 32 threads holding 8.  The matrix instructions behind
+// it are v_mfma_f32_16x16x16_{f16,bf16} for one base tile of k and v_mfma_f32_16x16x32_* for
+// two adjacent ones.  WideBaseTileShape is the 16 x 32 operand block of the 16x16x32
+// instruction taken in one piece (an extension, see types/register.hpp).
 #pragma once
 
 #include <hip/hip_bf16.h>
@@ -37,17 +40,31 @@ struct AccessBase {
   static constexpr int kExpectedSize = kMemTransWidth / kElementBits;
 };
 
-// Shape of the tile one MFMA base tile of `Element`s covers, in its contiguous orientation:
-// 16 x 32 for 16-bit operands (16 x 16 x 32 instruction), 16 x 16 for fp32 accumulators.
-// For a column-major operand the roles of rows and columns swap (32 x 16).
+// The block of a matrix one base tile covers: 16 x 16 for every element type, operands and
+// accumulators alike (include/types/base.hpp:62-68).
 template <typename Element>
   requires BaseType<Element>
 struct BaseTileShape {
   static constexpr int kRows = 16;
-  static constexpr int kCols = sizeof(Element) == 2 ? 32 : 16;
+  static constexpr int kCols = 16;
   static constexpr int kNumel = kRows * kCols;
   static constexpr int kNumelPerLane = kNumel / WARP_SIZE;
 };
+
+// The 16 x 32 block (in its contiguous orientation; 32 x 16 for a column-major operand) a
+// wide 16-bit operand base tile covers.
+template <typename Element>
+  requires HalfType<Element>
+struct WideBaseTileShape {
+  static constexpr int kRows = 16;
+  static constexpr int kCols = 32;
+  static constexpr int kNumel = kRows * kCols;
+  static constexpr int kNumelPerLane = kNumel / WARP_SIZE;
+};
+
+// Kernels written against earlier revisions of the reference spell traits::BaseTileShape (its
+// own examples/101_gemm still do); the name resolves here.
+namespace traits = ::tilefusion;
 
 template <typename T>
 HOST_DEVICE T from_float(float v) {

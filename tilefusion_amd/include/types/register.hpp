@@ -1,14 +1,20 @@
-// Register tiles (counterpart of include/types/register.hpp:84-131), re-sized for CDNA4.
+// Register tiles (counterpart of include/types/register.hpp:84-131) on a 64-lane wavefront.
 //
 // A RegTile is a per-lane array; a RegTile OF RegTiles tiles a wavefront-level matrix with
-// MFMA base tiles.  For v_mfma_f32_16x16x32_{f16,bf16} a lane l of the 64 holds
-//   * row-major operand base tile (16 rows x 32 k):   row l%16, k = 8*(l/16) .. +7   -> 1 x 8
-//   * col-major operand base tile (32 k x 16 cols):   col l%16, k = 8*(l/16) .. +7   -> 8 x 1
-//   * accumulator base tile (16 x 16), row-major:     col l%16, rows 4*(l/16) .. +3  -> 4 x 1
-//   * accumulator base tile, column-major view:       row l%16, cols 4*(l/16) .. +3  -> 1 x 4
-// BaseTileRowMajor<T> / BaseTileColMajor<T> pick the operand tile for 16-bit T and the
-// accumulator tile for float; BaseTileAccRowMajor<T> is the accumulator tile for any T (e.g.
-// scores converted to fp16 before they are stored).
+// base tiles.  A base tile covers the reference's 16 x 16 block; lane l of the 64 holds
+//   * BaseTileRowMajor<T> = RegTile<T, RowMajor<1, 4>>:  row l%16,    columns 4*(l/16) .. +3
+//   * BaseTileColMajor<T> = RegTile<T, ColMajor<4, 1>>:  column l%16, rows    4*(l/16) .. +3
+// for every element type.  These are the A and B operand layouts of v_mfma_*_16x16x16 (two
+// tiles adjacent in k feed one 16x16x32 instruction, see cell/compute/gemm.hpp), and the
+// row-major tile is also the layout of an accumulator block computed with the two operands
+// swapped - so, as with the reference's mma.m16n8k16 tiles, the accumulator of one gemm()
+// becomes the A operand of the next after an element-wise conversion, and the same
+// BaseTileRowMajor<float> the reference's kernels declare their accumulators with works here.
+//
+// Extension: a wide operand tile takes the whole 16 x 32 (32 x 16) block of the 16x16x32
+// instruction in one piece, one 16-byte access per lane:
+//   * WideBaseTileRowMajor<T> = RegTile<T, RowMajor<1, 8>>:  row l%16,    columns 8*(l/16) .. +7
+//   * WideBaseTileColMajor<T> = RegTile<T, ColMajor<8, 1>>:  column l%16, rows    8*(l/16) .. +7
 #pragma once
 
 #include "types/layout.hpp"
@@ -61,29 +67,41 @@ class RegTile {
 };
 
 template <typename T>
-inline constexpr bool kIsOperandType = sizeof(T) == 2;
-
+using BaseTileRowMajor = RegTile<T, tl::RowMajor<1, 4>>;
 template <typename T>
-using BaseTileRowMajor =
-    std::conditional_t<kIsOperandType<T>, RegTile<T, tl::RowMajor<1, 8>>, RegTile<T, tl::RowMajor<4, 1>>>;
+using BaseTileColMajor = RegTile<T, tl::ColMajor<4, 1>>;
 template <typename T>
-using BaseTileColMajor =
-    std::conditional_t<kIsOperandType<T>, RegTile<T, tl::ColMajor<8, 1>>, RegTile<T, tl::ColMajor<1, 4>>>;
+  requires HalfType<T>
+using WideBaseTileRowMajor = RegTile<T, tl::RowMajor<1, 8>>;
 template <typename T>
-using BaseTileAccRowMajor = RegTile<T, tl::RowMajor<4, 1>>;
-template <typename T>
-using BaseTileAccColMajor = RegTile<T, tl::ColMajor<1, 4>>;
+  requires HalfType<T>
+using WideBaseTileColMajor = RegTile<T, tl::ColMajor<8, 1>>;
 
 // What a base tile covers at wavefront level, from its per-lane shape.
 template <typename BaseTile>
 struct BaseTileTraits {
   using DType = typename BaseTile::DType;
-  static constexpr bool kIsOperand = BaseTile::kNumel == 8;
-  static constexpr bool kIsRowMajor = BaseTile::kType == tl::Layout::kRowMajor;
-  static_assert(BaseTile::kNumel == 8 || BaseTile::kNumel == 4, "not an MFMA base tile");
+  static_assert((BaseTile::kRows == 1 && (BaseTile::kCols == 4 || BaseTile::kCols == 8)) ||
+                    (BaseTile::kCols == 1 && (BaseTile::kRows == 4 || BaseTile::kRows == 8)),
+                "not a base tile: use BaseTileRowMajor / BaseTileColMajor (or the wide forms)");
+  static constexpr bool kIsWide = BaseTile::kNumel == 8;
+  // a lane owns (part of) a row of the block, or (part of) a column
+  static constexpr bool kIsRowMajor = BaseTile::kRows == 1;
+  static constexpr int kNumelPerLane = BaseTile::kNumel;
   // rows x cols of the matrix block one base tile holds across the 64 lanes
-  static constexpr int kRows = kIsOperand ? (kIsRowMajor ? 16 : 32) : 16;
-  static constexpr int kCols = kIsOperand ? (kIsRowMajor ? 32 : 16) : 16;
+  static constexpr int kRows = kIsRowMajor ? 16 : 4 * kNumelPerLane;
+  static constexpr int kCols = kIsRowMajor ? 4 * kNumelPerLane : 16;
+
+  // (row, col) inside the block of per-lane element e of lane `lane`
+  DEVICE static void coord(int lane, int e, int& r, int& c) {
+    if constexpr (kIsRowMajor) {
+      r = lane % 16;
+      c = kNumelPerLane * (lane / 16) + e;
+    } else {
+      r = kNumelPerLane * (lane / 16) + e;
+      c = lane % 16;
+    }
+  }
 };
 
 }  // namespace tilefusion

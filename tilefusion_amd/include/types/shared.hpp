@@ -38,6 +38,12 @@ class SharedTile {
   static constexpr int kSwizzleRows = isRowMajor ? SwizzleBaseShape::kRows : SwizzleBaseShape::kCols;
   static constexpr int kSwizzleCols = isRowMajor ? SwizzleBaseShape::kCols : SwizzleBaseShape::kRows;
 
+  // the swizzle permutes 16-byte vectors inside kSwizzleCols-wide blocks of a row (column):
+  // the contiguous extent of the (parent) tile must be whole blocks
+  static_assert(!kSwizzled || (isRowMajor ? kRowStride : kColStride) % kSwizzleCols == 0,
+                "a swizzled tile's contiguous dimension must be a multiple of the swizzle width "
+                "(SwizzleBytes / sizeof(element))");
+
   DEVICE SharedTile() : data_(nullptr), offset_(0) {}
   DEVICE SharedTile(DType* data) : data_(data), offset_(0) {}
   DEVICE SharedTile(const DType* data) : data_(const_cast<DType*>(data)), offset_(0) {}
