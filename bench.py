@@ -14,13 +14,18 @@ Timing: W untimed warm-up steps, then exactly K steps between two HIP events rec
 stream the kernels are launched on, bracketed by torch.cuda.synchronize().  Input sets rotate
 so that consecutive launches do not hit the 256 MB last-level cache with the same operands.
 The roofline entry is algorithmic flops (or bytes) per launch divided by the measured average
-launch duration.  The CPU baseline is the fp32 torch oracle timed on this host.
+launch duration; its "traffic" is read from the rocprofv3 summary of the workload under profiles/
+(counter runs are separate processes).  A second, separate pass times every step with its own
+event pair and reports the fastest and the median step next to the mean.  The CPU baseline is the
+fp32 torch oracle timed on this host.
 """
 
 import argparse
 import json
 import math
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -64,6 +69,33 @@ def _time_steps(fn, steps, warmup, pre_warm_ms=PRE_WARM_MS):
     return e0.elapsed_time(e1) / steps, wall / steps
 
 
+def _time_each_step(fn, steps, first):
+    """Fastest and median of `steps` individually timed steps (one event pair each; the pairs add
+    a few microseconds of launch gap, so these figures are reported next to the mean of the
+    back-to-back region, they do not replace it)."""
+    import torch
+    pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for i, (e0, e1) in enumerate(pairs):
+        e0.record()
+        fn(first + i)
+        e1.record()
+    torch.cuda.synchronize()
+    t = [e0.elapsed_time(e1) for e0, e1 in pairs]
+    return min(t), statistics.median(t)
+
+
+def _profile_traffic(name):
+    """Bytes per step between the L2 caches and the fabric, as the rocprofv3 summary of the workload
+    states them (FETCH_SIZE + WRITE_SIZE per launch, each scaled by what the counter reads for a
+    1 GiB copy); None when the summary is missing or does not carry the figure."""
+    try:
+        text = open(os.path.join(ROOT, "profiles", name + ".txt")).read()
+    except OSError:
+        return None
+    m = re.search(r"scaled traffic per step:.*\((\d+) bytes\)", text)
+    return int(m.group(1)) if m else None
+
+
 def _bound_calls(fn, arg_lists, err):
     """One closure per operand set with every argument already converted: a step is then a
     single C call, so that the host side of a step stays well under a few-microsecond kernel."""
@@ -79,25 +111,25 @@ def _bound_calls(fn, arg_lists, err):
     return [make(a) for a in arg_lists]
 
 
-def _cpu_time(fn, reps=3):
-    fn()
-    best = float("inf")
+def _cpu_times(fn, reps=3, warm=True):
+    """(best, median) wall time of `reps` calls, after one untimed call when `warm`."""
+    if warm:
+        fn()
+    t = []
     for _ in range(reps):
         t0 = time.perf_counter()
         fn()
-        best = min(best, time.perf_counter() - t0)
-    return best
+        t.append(time.perf_counter() - t0)
+    return min(t), statistics.median(t)
 
 
 class Gemm4096:
     name = "gemm_fp16_4096x4096x4096"
+    profile = "gemm_fp16_4096"   # profiles/<this>.txt
     metric, unit, bound = "gemm_fp16_tflops", "TFLOP/s", "mfma"
     M = N = K = 4096
     flops = 2.0 * 4096 ** 3
     bytes = 3 * 4096 * 4096 * 2
-    # Measured bytes per launch between the L2 caches and the fabric (rocprofv3 FETCH_SIZE +
-    # WRITE_SIZE, each scaled by what it reads for a 1 GiB copy; summaries under profiles/).
-    traffic = 235087049
 
     def setup(self, dev):
         import torch
@@ -128,8 +160,9 @@ class Gemm4096:
     def cpu_baseline(self):
         import torch
         a32, b32 = self.host[0].float(), self.host[1].float()
-        t = _cpu_time(lambda: torch.matmul(a32, b32.T))
-        return {"value": self.flops / t / 1e12, "unit": "TFLOP/s", "sample": "full 4096^3 fp32 torch.matmul, best of 3"}
+        best, med = _cpu_times(lambda: torch.matmul(a32, b32.T))
+        return {"value": self.flops / best / 1e12, "median": self.flops / med / 1e12, "unit": "TFLOP/s",
+                "sample": "full 4096^3 fp32 torch.matmul, 1 warm-up + 3 repetitions (value = best, median beside it)"}
 
     config = {"workload": "fp16 GEMM M=N=K=4096, A row-major, B col-major, fp32 accumulate, fp16 out",
               "inputs": "N(0,1)/sqrt(K), seed 1002; 4 rotating operand sets"}
@@ -141,7 +174,6 @@ class Fused:
     M, N, K, P = 16384, 128, 128, 128
     flops = 2.0 * 2 * 16384 * 128 * 128
     bytes = (16384 * 128 * 2 + 2 * 128 * 128) * 2
-    traffic = 9067224  # measured, see Gemm4096.traffic
 
     def setup(self, dev):
         import torch
@@ -168,8 +200,9 @@ class Fused:
 
     def cpu_baseline(self):
         a, b, c = (t.float() for t in self.host)
-        t = _cpu_time(lambda: (a @ b.T) @ c.T)
-        return {"value": self.bytes / t / 1e9, "unit": "GB/s", "sample": "full problem, two fp32 torch.matmul, best of 3"}
+        best, med = _cpu_times(lambda: (a @ b.T) @ c.T)
+        return {"value": self.bytes / best / 1e9, "median": self.bytes / med / 1e9, "unit": "GB/s",
+                "sample": "full problem, two fp32 torch.matmul, 1 warm-up + 3 repetitions (value = best, median beside it)"}
 
     config = {"workload": "fused (A[16384x128] @ B[128x128]) @ C[128x128], fp16 in/out, fp32 accumulate",
               "inputs": "N(0,1)/sqrt(128), seed 1003; 40 rotating A/D sets"}
@@ -185,7 +218,6 @@ class Attention:
         self.metric = "flash_attention_fwd_tflops" + ("_causal" if causal else "")
         self.flops = 4.0 * 64 * 4096 * 4096 * 128 * (0.5 if causal else 1.0)
         self.bytes = 4 * 64 * 4096 * 128 * 2
-        self.traffic = 384216579 if causal else 268700488  # measured, see Gemm4096.traffic
         self.config = {"workload": "flash-attention fwd fp16 B=2 H=32 S=4096 D=128 %s, scale 1/sqrt(128), fp32 softmax stats"
                        % ("causal" if causal else "non-causal"),
                        "inputs": "N(0,1), seed 1004; V in natural [S, D] layout; 2 rotating Q/K/V/O sets"}
@@ -224,14 +256,19 @@ class Attention:
     def cpu_baseline(self):
         import oracle
         q, k, v = self.host
-        n = len(self._sample)
-
-        def run():
-            for b, h in self._sample:
+        oracle.attention_ref(q[0, 0], k[0, 0], v[0, 0], causal=self.causal)   # untimed warm-up slice
+        per_slice = []
+        for b in range(self.B):
+            for h in range(self.H):
+                t0 = time.perf_counter()
                 oracle.attention_ref(q[b, h], k[b, h], v[b, h], causal=self.causal)
-        t = _cpu_time(run, reps=2)
-        return {"value": self.flops * n / 64 / t / 1e12, "unit": "TFLOP/s",
-                "sample": "extrapolated from %d of 64 (batch, head) slices (rate = sampled flops / sampled time), fp32 softmax(QK^T)V per slice, best of 2" % n}
+                per_slice.append(time.perf_counter() - t0)
+        total = sum(per_slice)
+        per = self.flops / 64
+        return {"value": self.flops / total / 1e12, "unit": "TFLOP/s",
+                "best_slice": per / min(per_slice) / 1e12, "median_slice": per / statistics.median(per_slice) / 1e12,
+                "sample": "all 64 (batch, head) slices, one repetition after one warm-up slice: fp32 softmax(QK^T)V per "
+                          "slice (value = whole-workload flops / total time; rate of the best and of the median slice beside it)"}
 
 
 class Decode:
@@ -240,7 +277,6 @@ class Decode:
     BH, LKV, D, SPLITS = 512, 32768, 128, 64
     bytes = 2 * 512 * 32768 * 128 * 2 + 2 * 512 * 128 * 2
     flops = 4.0 * 512 * 32768 * 128
-    traffic = 8626347552  # both kernels of a step; measured, see Gemm4096.traffic
 
     def setup(self, dev):
         import torch
@@ -264,6 +300,7 @@ class Decode:
         self.calls[0]()
 
     _sample = [0, 100, 255, 511]
+    _cpu_slices = 64
 
     def check(self):
         import oracle
@@ -276,14 +313,20 @@ class Decode:
 
     def cpu_baseline(self):
         import oracle
-        host = [(self.q[i].cpu(), self.k[i].cpu(), self.v[i].cpu()) for i in self._sample]
-
-        def run():
-            for q, k, v in host:
-                oracle.flash_decode_ref(q, k, v)
-        t = _cpu_time(run)
-        return {"value": self.bytes * len(host) / self.BH / t / 1e9, "unit": "GB/s",
-                "sample": "extrapolated from %d of 512 (batch, head) slices (rate = sampled bytes / sampled time), fp32 softmax(qK^T)V per slice, best of 3" % len(host)}
+        idx = list(range(0, self.BH, self.BH // self._cpu_slices))
+        per_slice = []
+        for n, i in enumerate([idx[0]] + idx):   # the first one twice: warm-up
+            q, k, v = self.q[i].cpu(), self.k[i].cpu(), self.v[i].cpu()
+            t0 = time.perf_counter()
+            oracle.flash_decode_ref(q, k, v)
+            if n:
+                per_slice.append(time.perf_counter() - t0)
+        per = self.bytes / self.BH
+        return {"value": per * len(idx) / sum(per_slice) / 1e9, "unit": "GB/s",
+                "best_slice": per / min(per_slice) / 1e9, "median_slice": per / statistics.median(per_slice) / 1e9,
+                "sample": "%d of 512 (batch, head) slices (every 8th), one repetition after one warm-up slice: fp32 "
+                          "softmax(qK^T)V per slice with K, V upcast per slice (value = sampled bytes / sampled time; "
+                          "rate of the best and of the median slice beside it)" % len(idx)}
 
     config = {"workload": "flash-decoding fp16 B=16 H=32 q_len=1 KV=32768 D=128, 64 splits + LSE combine (2 kernels per step)",
               "inputs": "N(0,1) drawn on the device, seed 1005; 8 GiB of K,V (exceeds the last-level cache)"}
@@ -326,6 +369,7 @@ def run_workload(w, steps, warmup, with_cpu, pre_warm_ms=PRE_WARM_MS):
     w.setup(dev)
     ok, rel, mabs = w.check()
     ms, wall_ms = _time_steps(w.step, steps, warmup, pre_warm_ms)
+    step_min, step_median = _time_each_step(w.step, steps, warmup + steps)
     if w.bound == "mfma":
         achieved, peak, runit = w.flops / ms / 1e9, PEAK_FP16_TFLOPS, "TFLOP/s"
     else:
@@ -333,8 +377,10 @@ def run_workload(w, steps, warmup, with_cpu, pre_warm_ms=PRE_WARM_MS):
     out = {
         "metric": w.metric, "value": round(achieved, 2), "unit": w.unit, "ms_per_step": round(ms, 5),
         "wall_ms_per_step": round(wall_ms, 5),
+        "step_ms_individually_timed": {"min": round(step_min, 5), "median": round(step_median, 5)},
         "roofline": {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": runit,
-                     "frac": round(achieved / peak, 4), "traffic": getattr(w, "traffic", None)},
+                     "frac": round(achieved / peak, 4),
+                     "traffic": None if isinstance(w, Copy) else _profile_traffic(getattr(w, "profile", w.name))},
         "tflops": round(w.flops / ms / 1e9, 2), "algorithmic_gbs": round(w.bytes / ms / 1e6, 1),
         "parity": {"ok": bool(ok), "rel_l2": float("%.3e" % rel), "max_abs": float("%.3e" % mabs),
                    "tolerance": "rel_l2<=1e-3, max_abs<=2e-2 vs fp32 CPU oracle"},
@@ -342,7 +388,9 @@ def run_workload(w, steps, warmup, with_cpu, pre_warm_ms=PRE_WARM_MS):
     }
     if with_cpu:
         cb = w.cpu_baseline()
-        cb["value"] = round(cb["value"], 4)
+        for key in ("value", "median", "best_slice", "median_slice"):
+            if key in cb:
+                cb[key] = round(cb[key], 4)
         cb["cores"] = torch.get_num_threads()
         cb["kind"] = "port"
         out["cpu_baseline"] = cb
@@ -382,6 +430,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic", "config": head["config"], "roofline": head["roofline"],
         "parity": head["parity"],
+        "step_ms_individually_timed": head["step_ms_individually_timed"],
         "device": {"name": prop.name, "cus": prop.multi_processor_count, "host_cores": os.cpu_count()},
     }
     if "cpu_baseline" in head:

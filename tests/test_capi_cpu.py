@@ -117,3 +117,16 @@ def test_reference_package_name_imports_the_same_modules():
     assert tilefusion.ops is tilefusion_amd.ops
     assert gemm is tilefusion_amd.ops.gemm and fused_two_gemms is tilefusion_amd.ops.fused_two_gemms
     assert flash_attention is tilefusion_amd.ops.flash_attention
+
+
+def test_torch_binding_exports_the_reference_launcher_names():
+    # TILEFUSION_EXPORT (include/kernel_registry.hpp:20-24, include/kernels/ops.hpp:36-58): the four host
+    # launchers are C-linkage symbols of libtilefusion.so under the reference's names
+    import ctypes
+    import os
+
+    import torch  # noqa: F401  (the binding links against libtorch)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    lib = ctypes.CDLL(os.path.join(root, "tilefusion_amd", "libtilefusion.so"))
+    for name in ("gemm", "fused_two_gemms", "flash_attention", "scatter_nd"):
+        assert hasattr(lib, name), name

@@ -229,9 +229,12 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       const char* base = r < kKPerWave ? reinterpret_cast<const char*>(K + (size_t)n0 * D)
                          : kVT         ? reinterpret_cast<const char*>(V + n0)
                                        : reinterpret_cast<const char*>(V + (size_t)n0 * DV);
-      asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+      // the LDS destination is an M0 INPUT of the statement: the compiler writes M0 itself and
+      // cannot use the register for anything else between that write and the request; the
+      // s_nop is the wait state an M0 write needs in front of an LDS-direct load
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                    :
-                   : "v"(req_off[r]), "s"(base), "s"(dst)
+                   : "v"(req_off[r]), "s"(base), "{m0}"(dst)
                    : "memory");
       return;
     }
@@ -267,9 +270,9 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     const char* base = r < kKPerWave ? reinterpret_cast<const char*>(K) + (size_t)tile * (kBN * D * 2)
                        : kVT         ? reinterpret_cast<const char*>(V) + (size_t)tile * (kBN * 2)
                                      : reinterpret_cast<const char*>(V) + (size_t)tile * (kBN * DV * 2);
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(req_off[r]), "s"(base), "s"(dst)
+                 : "v"(req_off[r]), "s"(base), "{m0}"(dst)
                  : "memory");
   };
   auto issue_tile_loads = [&](int tile) __attribute__((always_inline)) {

@@ -185,9 +185,12 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
   const unsigned a_off = ((unsigned)a_row * (unsigned)K + 8u * lg) * 2u;
   const unsigned sB_addr = lds_address(sB), sC_addr = lds_address(sC);
   auto dma = [](unsigned off, const char* base, unsigned lds_addr) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+    // the LDS destination is an M0 INPUT of the statement: the compiler writes M0 itself and
+    // cannot use the register for anything else between that write and the request; the s_nop
+    // is the wait state an M0 write needs in front of an LDS-direct load
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
-                 : "v"(off), "s"(base), "s"(lds_addr)
+                 : "v"(off), "s"(base), "{m0}"(lds_addr)
                  : "memory");
   };
 
@@ -456,20 +459,22 @@ __global__ __launch_bounds__(kWavesT * kSplit * 64) void fused_two_gemms_stream_
       const int i_first = wave_id * (kBInstr / kReqWaves);
       const unsigned voff = voff_b0 ^ (unsigned)(((q % 4) * 4) << 4);        // row 4i: chunk ^= 4 * (i % 4)
       const char* src = b_src + (size_t)(i_first + q) * 1024 - (q % 4) * 1024;   // + rows, - what the immediate adds
-      if (q % 4 == 0)
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(src), "s"(stage + (i_first + q) * 1024) : "memory");
-      else
-        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(src), "n"(1024 * (q % 4)) : "memory");
+      // four requests share one M0 value (an input of each statement, so the compiler keeps it
+      // there) and differ in the immediate offset
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2"
+                   :
+                   : "v"(voff), "s"(src), "n"(1024 * (q % 4)), "{m0}"(stage + (i_first + q - q % 4) * 1024)
+                   : "memory");
     }
 #pragma unroll
     for (int q = 0; q < kCInstr / kReqWaves; ++q) {
       const int i_first = wave_id * (kCInstr / kReqWaves);
       const unsigned voff = voff_c0 ^ (unsigned)(((q % 2) * 4) << 4);        // row 8i: chunk ^= 4 * (i % 2)
       const char* src = c_src + (size_t)(i_first + q) * 8 * (size_t)N * 2 - (q % 4) * 1024;
-      if (q % 4 == 0)
-        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(src), "s"(stage + kBBytes + (i_first + q) * 1024) : "memory");
-      else
-        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(src), "n"(1024 * (q % 4)) : "memory");
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2"
+                   :
+                   : "v"(voff), "s"(src), "n"(1024 * (q % 4)), "{m0}"(stage + kBBytes + (i_first + q - q % 4) * 1024)
+                   : "memory");
     }
   };
 

@@ -27,6 +27,11 @@ using __bfloat16 = at::BFloat16;
 
 namespace tilefusion {
 
+// Marks the host launchers the Python side binds (include/kernel_registry.hpp:20-24): C linkage and
+// default visibility, so `gemm`, `fused_two_gemms`, `flash_attention` and `scatter_nd` are exported
+// from libtilefusion.so under the names the reference's library exports them.
+#define TILEFUSION_EXPORT extern "C" __attribute__((visibility("default")))
+
 #define CHECK_CUDA(x) TORCH_CHECK((x).device().is_cuda(), #x " must be a CUDA tensor.")
 #define CHECK_CONTIGUOUS(x) TORCH_CHECK((x).is_contiguous(), #x " must be contiguous.")
 #define CHECK_INPUT(x) \
@@ -75,7 +80,7 @@ int64_t leading_numel(const at::Tensor& t, int64_t keep) {
 namespace kernels {
 
 // gemm(A [M,K], B [N,K] (= column-major K x N), C [M,N] fp32 or fp16)
-void gemm(const at::Tensor& A, const at::Tensor& B, at::Tensor& C, int64_t tm, int64_t tn,
+TILEFUSION_EXPORT void gemm(const at::Tensor& A, const at::Tensor& B, at::Tensor& C, int64_t tm, int64_t tn,
           int64_t tk, int64_t num_stages, int64_t pipeline_level) {
   CHECK_INPUT(A);
   CHECK_INPUT(B);
@@ -96,7 +101,7 @@ void gemm(const at::Tensor& A, const at::Tensor& B, at::Tensor& C, int64_t tm, i
 }
 
 // fused_two_gemms(A [.., M,K], B [.., N,K], C [.., P,N], D [.., M,P])
-void fused_two_gemms(const at::Tensor& A, const at::Tensor& B, const at::Tensor& C, at::Tensor& D,
+TILEFUSION_EXPORT void fused_two_gemms(const at::Tensor& A, const at::Tensor& B, const at::Tensor& C, at::Tensor& D,
                      int64_t tm, int64_t tn, int64_t tk, int64_t tp) {
   CHECK_INPUT(A);
   CHECK_INPUT(B);
@@ -231,7 +236,7 @@ void attention_impl(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& 
 
 // flash_attention(Q [.., Lq,D], K [.., Lkv,D], V [.., Dv,Lkv] (transposed, as the reference's
 // Python wrapper passes it), O [.., Lq,Dv])
-void flash_attention(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V, at::Tensor& O,
+TILEFUSION_EXPORT void flash_attention(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V, at::Tensor& O,
                      int64_t tile_length_q, int64_t tile_length_kv, int64_t tile_hidden_qk,
                      int64_t tile_hidden_v, double softmax_scale, bool causal) {
   attention_impl(Q, K, V, O, true, tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v,
@@ -275,7 +280,7 @@ void flash_decode(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V,
 // scatter_nd(data [d0..dr-1], updates [n.., d_k..d_{r-1}], indices [n.., k] int64): data[idx] += updates.
 // The reference's schema marks `updates` as the mutated tensor although its kernel writes
 // `data` (src/kernels/scatter_nd.cu:86-92); the schema is kept, `data` is what changes.
-void scatter_nd(const at::Tensor& data, at::Tensor& updates, const at::Tensor& indices) {
+TILEFUSION_EXPORT void scatter_nd(const at::Tensor& data, at::Tensor& updates, const at::Tensor& indices) {
   CHECK_INPUT(data);
   CHECK_INPUT(updates);
   CHECK_INPUT(indices);

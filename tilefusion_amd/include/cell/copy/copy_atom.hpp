@@ -37,9 +37,12 @@ DEVICE void ld_shared_st_global(void* global_dst, const void* shared_src) {
 DEVICE void ld_global_direct_to_shared_16B(unsigned lds_wave_base, const void* global_src) {
   // readfirstlane: the value is uniform by contract, this makes it a scalar register by type
   const unsigned base = __builtin_amdgcn_readfirstlane(lds_wave_base);
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+  // M0 (the LDS destination) is an INPUT of the statement: the compiler writes it and cannot use
+  // the register for anything else between that write and the load; the s_nop is the wait state
+  // an M0 write needs in front of an LDS-direct load
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
-               : "v"(global_src), "s"(base)
+               : "v"(global_src), "{m0}"(base)
                : "memory");
 }
 // LDS byte address of a pointer into LDS (what M0 takes).
