@@ -54,9 +54,12 @@ TFK_DEVICE void load_global_to_lds_16B(const void* gptr, void* lds_wave_base) {
 // the caller's job (wait_vmem / barrier_keep_vmem below).  `lds_addr` is the wave-uniform LDS
 // byte address of the 1 KiB destination.
 TFK_DEVICE void lds_dma_16B(const void* gptr, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+  // M0 (the LDS destination) is an INPUT of the statement: the compiler writes it and cannot use the
+  // register for anything else between that write and the load; the s_nop is the wait state an
+  // M0 write needs in front of an LDS-direct load
+  asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
-               : "v"(gptr), "s"(lds_addr)
+               : "v"(gptr), "{m0}"(lds_addr)
                : "memory");
 }
 TFK_DEVICE unsigned lds_address(const void* p) {

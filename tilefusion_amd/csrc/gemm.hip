@@ -405,18 +405,8 @@ struct Ring64Shape {
   }
   static_assert((TM == 8 || TM == 4) && (TN == 8 || TN == 4) && TM % kLoads == 0 && kLoads % 4 == 0,
                 "slot schedule: a request every TM / kLoads slots, M0 shared by four requests");
-  // M0 is written in the last gap of the slot in front of requests 0, 4, ...
-  static constexpr bool m0_slot_after(int i) {
-    const int i_next = (i + 1) % TM;
-    return i_next % (TM / kLoads) == 0 && (i_next / (TM / kLoads)) % 4 == 0;
-  }
-  static constexpr bool m0_gaps_free() {
-    for (int i = 0; i < TM; ++i)
-      if (m0_slot_after(i) && gap_has_read(i, TN - 1)) return false;
-    return true;
-  }
-  static_assert(reads_fit() && free_gaps() >= 7 && m0_gaps_free(),
-                "slot schedule: every read, bookkeeping piece and M0 write needs its own gap");
+  static_assert(reads_fit() && free_gaps() >= 7,
+                "slot schedule: every read and bookkeeping piece needs its own gap");
   static_assert((2 * kAhead - 3) * kLoads < 64, "vmcnt is a 6-bit counter");
   // 128-byte rows: two rows per pass over the banks; chunk ^ (row / 2) % 8 keeps every
   // ds_read_b128 lane pass on 16 different bank groups
@@ -479,13 +469,16 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   // and the vector-memory waits are placed by hand below.
   // src: tile origin + k offset (scalar); lds_unit: LDS byte address of this wavefront's first
   // 1 KiB block in the destination unit.
-  // M0 (the LDS destination of requests n .. n+3, n % 4 == 0) is written one MFMA gap ahead of
-  // the first of them, which saves the wait state an M0 write needs in front of its use.
-  auto set_m0 = [&](unsigned lds_unit, int n) __attribute__((always_inline)) {
-    asm volatile("s_mov_b32 m0, %0" : : "s"(lds_unit + n * 1024) : "memory");
-  };
-  auto request = [&](const char* src, int n) __attribute__((always_inline)) {
-    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(g_off[n]), "s"(src), "n"(1024 * (n % 4)) : "memory");
+  // M0 - the LDS destination of requests n .. n+3 (n % 4 == 0), which differ in the immediate
+  // offset - is an INPUT of every request statement: the compiler writes it (once per group of
+  // four: the statements do not change it) and cannot use the register for anything else between
+  // that write and a request.  The s_nop is the wait state an M0 write needs in front of an
+  // LDS-direct load; next to a request at the head of a slot it costs no issue time.
+  auto request = [&](const char* src, unsigned lds_unit, int n) __attribute__((always_inline)) {
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2"
+                 :
+                 : "v"(g_off[n]), "s"(src), "n"(1024 * (n % 4)), "{m0}"(lds_unit + (n - n % 4) * 1024)
+                 : "memory");
   };
   auto k_src = [&](const char* tile, int t) __attribute__((always_inline)) {
     return tile + (size_t)min(t, num_k_tiles - 1) * S::BK * 2;   // clamped past the end
@@ -544,11 +537,7 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
   for (int u = 0; u < 2 * S::kAhead; ++u)
 #pragma unroll
     for (int n = 0; n < S::kLoads; ++n) {
-      if (n % 4 == 0) {
-        set_m0(lds_wave + u * S::kUnitBytes, n);
-        asm volatile("s_nop 0");
-      }
-      request(k_src(u % 2 ? b_tile : a_tile, u / 2), n);
+      request(k_src(u % 2 ? b_tile : a_tile, u / 2), lds_wave + u * S::kUnitBytes, n);
     }
   wait_vmem<2 * (S::kAhead - 1) * S::kLoads>();
   __builtin_amdgcn_s_barrier();
@@ -614,24 +603,14 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  // request n of a k-step goes at the head of slot n * kSlotsPerLoad; if n % 4 == 0 its M0 is
-  // written in the last gap of the slot before (for slot 0: of the previous k-step's slot 7)
-  auto m0_slot = [&](int i, int j, unsigned next_unit, unsigned this_unit) __attribute__((always_inline)) {
-    if (j != S::TN - 1 || !S::m0_slot_after(i)) return;
-    const int i_next = (i + 1) % S::TM;
-    __builtin_amdgcn_sched_barrier(0);
-    set_m0(i_next == 0 ? next_unit : this_unit, i_next / kSlotsPerLoad);
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  set_m0(req_a, 0);
+  // request n of a k-step goes at the head of slot n * kSlotsPerLoad
   for (int t = 0; t < num_k_tiles; ++t) {
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) request(src_a, i / kSlotsPerLoad);
+      if (i % kSlotsPerLoad == 0) request(src_a, req_a, i / kSlotsPerLoad);
       slot_pinned(0, i, rd_a1, rd_b1, [&](int j) __attribute__((always_inline)) {
         prep0(S::kPrep.piece[i * S::TN + j], t);
-        m0_slot(i, j, req_b, req_a);
       });
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -639,10 +618,9 @@ __global__ __launch_bounds__(S::kThreads) void gemm_ring64_kernel(
 #pragma unroll
     for (int i = 0; i < S::TM; ++i) {
       __builtin_amdgcn_sched_barrier(0);
-      if (i % kSlotsPerLoad == 0) request(src_b, i / kSlotsPerLoad);
+      if (i % kSlotsPerLoad == 0) request(src_b, req_b, i / kSlotsPerLoad);
       slot_pinned(1, i, rd_a0, rd_b0, [&](int j) __attribute__((always_inline)) {
         prep1(S::kPrep.piece[i * S::TN + j], t);
-        m0_slot(i, j, req_a, req_b);
       });
     }
     // The compiler does not know that the accumulators are written by MFMAs (they are issued
