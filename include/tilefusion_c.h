@@ -123,7 +123,7 @@ TF_API int tf_flash_attention_fwd(const void* Q, const void* K, const void* V, v
 /* Single-query (decoding) attention with the KV range split into `num_splits` chunks:
  * kernel 1 writes per-split partial (o, max, sum) in fp32 into `workspace`, kernel 2 merges
  * them with a log-sum-exp weighted sum into O.
- * Q [batch_heads, D]; K, V [batch_heads, Lkv, D]; O [batch_heads, D]; D must be 128.
+ * Q [batch_heads, D]; K, V [batch_heads, Lkv, D]; O [batch_heads, D]; D must be 128 or 64.
  * All offsets are 64-bit (K alone has 2^31 elements at the benchmark size).
  * No counterpart in the reference (it has no decoding kernel); built on the same online
  * softmax algebra as include/kernels/flash_attention_device.cuh:257-301. */
@@ -132,6 +132,12 @@ TF_API int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void
                                void* workspace, size_t workspace_bytes, int64_t batch_heads,
                                int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
                                void* stream);
+/* The same for fp16 or bf16 (dtype as in tf_gemm; the 16-bit types of the reference's dispatch,
+ * include/kernels/dispatch_macros.hpp:6-23): bf16 inputs, bf16 output, fp32 partials. */
+TF_API int tf_flash_decode(const void* Q, const void* K, const void* V, void* O, int dtype,
+                           void* workspace, size_t workspace_bytes, int64_t batch_heads,
+                           int64_t Lkv, int64_t D, int num_splits, double softmax_scale,
+                           void* stream);
 
 /* tf_flash_decode_f16 without the workspace argument and without any allocation: the per-split
  * partials live in a static device array inside the library (TF_FLASH_DECODE_STATIC_MAX_PARTIALS
@@ -140,7 +146,7 @@ TF_API int tf_flash_decode_f16(const void* Q, const void* K, const void* V, void
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The device that
  * owns `stream` must be current.  The first call on a device looks up the array's address there
  * (hipGetSymbolAddress); no call allocates or frees.  batch_heads * num_splits above
- * TF_FLASH_DECODE_STATIC_MAX_PARTIALS is rejected with TF_ERR_INVALID_ARG.  Same kernels and
+ * TF_FLASH_DECODE_STATIC_MAX_PARTIALS is rejected with TF_ERR_INVALID_ARG; D must be 128.  Same kernels and
  * bit-identical results as tf_flash_decode_f16.  All calls on one GPU share the one array, so
  * calls that overlap on a GPU (different streams, or threads) race: serialise them. */
 #define TF_FLASH_DECODE_STATIC_MAX_PARTIALS 32768 /* 512 (batch x head) slices x 64 splits */

@@ -95,13 +95,17 @@ def c_attention(q, k, v, causal=False, scale=None, v_transposed=False, tiles=Non
 
 
 def c_decode(q, k, v, num_splits, scale=None):
-    """q [BH, D], k, v [BH, Lkv, D]."""
+    """q [BH, D], k, v [BH, Lkv, D]; fp16 through tf_flash_decode_f16, bf16 through the dtype-coded entry."""
     lib = _capi.load()
     bh, lkv, d = k.shape
     scale = 1.0 / math.sqrt(d) if scale is None else scale
     nbytes = lib.tf_flash_decode_workspace_bytes(bh, d, num_splits)
     ws = torch.empty(nbytes, device=q.device, dtype=torch.uint8)
-    o = torch.full((bh, d), float("nan"), device=q.device, dtype=torch.float16)
-    _capi.check(lib.tf_flash_decode_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(), nbytes,
-                                        bh, lkv, d, num_splits, scale, stream()), "tf_flash_decode_f16")
+    o = torch.full((bh, d), float("nan"), device=q.device, dtype=q.dtype)
+    if q.dtype == torch.float16:
+        _capi.check(lib.tf_flash_decode_f16(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(), nbytes,
+                                            bh, lkv, d, num_splits, scale, stream()), "tf_flash_decode_f16")
+    else:
+        _capi.check(lib.tf_flash_decode(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), 2, ws.data_ptr(), nbytes,
+                                        bh, lkv, d, num_splits, scale, stream()), "tf_flash_decode")
     return o

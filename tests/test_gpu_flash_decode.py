@@ -31,6 +31,41 @@ def test_shapes_and_ragged_splits(bh, lkv, splits):
     assert ok, f"rel_l2={r:.3e} max_abs={m:.3e}"
 
 
+# The kernels are templates of the element type and the head dimension (the reference's 16-bit
+# types, include/kernels/dispatch_macros.hpp:6-23).  bf16: the oracle consumes the bf16-rounded
+# inputs in fp32, what is left is the rounding of the output to 8 mantissa bits (rel-L2 <= 4e-3,
+# max-abs <= 4e-2); head dimension 64 puts two key rows in a 16-lane group (8-lane reductions).
+@pytest.mark.parametrize("dtype,tol", [(torch.float16, (1e-3, 2e-2)), (torch.bfloat16, (4e-3, 4e-2))])
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("bh,lkv,splits", [(4, 1000, 3), (3, 5, 8), (2, 32768, 64), (5, 128, 128), (3, 257, 2),
+                                           (16, 4096, 16), (2, 2048, 1)])
+def test_element_types_and_head_dimensions(dtype, tol, d, bh, lkv, splits):
+    g = torch.Generator().manual_seed(bh * 100 + lkv + d)
+    q = torch.randn(bh, d, generator=g).to(dtype)
+    k = torch.randn(bh, lkv, d, generator=g).to(dtype)
+    v = torch.randn(bh, lkv, d, generator=g).to(dtype)
+    o = c_decode(q.to(DEV), k.to(DEV), v.to(DEV), splits)
+    assert o.dtype == dtype and not torch.isnan(o).any()
+    ref = N.flash_decode_ref(q, k, v, 1.0 / math.sqrt(d))
+    assert N.rel_l2(o, ref) <= tol[0] and N.max_abs(o, ref) <= tol[1], (N.rel_l2(o, ref), N.max_abs(o, ref))
+
+
+def test_one_hot_keys_pick_single_value_rows_exactly():
+    # a key that dominates by a wide margin makes the output that key's value row, bit for bit,
+    # in every type and head dimension (a wrong lane-group reduction or row mapping cannot hide)
+    for dtype in (torch.float16, torch.bfloat16):
+        for d in (64, 128):
+            g = torch.Generator().manual_seed(d)
+            bh, lkv = 6, 3000
+            q = torch.zeros(bh, d); q[:, 0] = 8.0
+            k = torch.zeros(bh, lkv, d)
+            hot = torch.randint(0, lkv, (bh,), generator=g)
+            k[torch.arange(bh), hot, 0] = 16.0          # logit 128 * scale against 0 everywhere else
+            v = torch.randint(-8, 9, (bh, lkv, d), generator=g).float()
+            o = c_decode(q.to(dtype).to(DEV), k.to(dtype).to(DEV), v.to(dtype).to(DEV), 7, 1.0)
+            assert torch.equal(o.float().cpu(), v[torch.arange(bh), hot]), (dtype, d)
+
+
 def test_scale_and_extreme_logits():
     q, k, v = _slices(4, 2048)
     for scale in (1.0, 1e-3, -0.2):

@@ -77,6 +77,21 @@ def test_flash_attention_batched_and_decode_ops():
     assert ok, (r, m)
 
 
+def test_flash_decode_op_takes_bf16_and_head_dimension_64():
+    from tilefusion_amd.ops import flash_decode
+    g = torch.Generator().manual_seed(31)
+    q = torch.randn(2, 4, 1, 64, generator=g).bfloat16()
+    k = torch.randn(2, 4, 1500, 64, generator=g).bfloat16()
+    v = torch.randn(2, 4, 1500, 64, generator=g).bfloat16()
+    o = flash_decode(q.to(DEV), k.to(DEV), v.to(DEV), num_splits=5)
+    assert o.shape == q.shape and o.dtype == torch.bfloat16
+    ref = N.flash_decode_ref(q.view(8, 64), k.view(8, 1500, 64), v.view(8, 1500, 64))
+    # bf16 output: 8 mantissa bits
+    assert N.rel_l2(o.view(8, 64), ref) <= 4e-3 and N.max_abs(o.view(8, 64), ref) <= 4e-2
+    with pytest.raises(RuntimeError, match="same dtype"):
+        flash_decode(q.to(DEV), k.half().to(DEV), v.to(DEV), num_splits=5)
+
+
 def test_ops_run_on_the_current_stream():
     from tilefusion_amd.ops import gemm
     a, b = oracle.make_c1_gemm_inputs(512, 512, 512)

@@ -257,10 +257,10 @@ void flash_decode(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V,
   CHECK_INPUT(K);
   CHECK_INPUT(V);
   CHECK_INPUT(O);
-  CHECK_HALF(Q);
-  CHECK_HALF(K);
-  CHECK_HALF(V);
-  CHECK_HALF(O);
+  CHECK_SAME_TYPE(Q, K);
+  CHECK_SAME_TYPE(Q, V);
+  CHECK_SAME_TYPE(Q, O);
+  const int dtype = operand_dtype(Q, "flash_decode");
   TORCH_CHECK(K.dim() >= 2 && V.dim() == K.dim(), "flash_decode: K and V must be [.., Lkv, D].");
   const int64_t d = K.size(-1), lkv = K.size(-2);
   const int64_t bh = leading_numel(K, 2);
@@ -271,9 +271,9 @@ void flash_decode(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& V,
   TORCH_CHECK(num_splits > 0, "flash_decode: num_splits must be positive.");
   const size_t bytes = tf_flash_decode_workspace_bytes(bh, d, (int)num_splits);
   at::Tensor ws = at::empty({(int64_t)((bytes + 3) / 4)}, Q.options().dtype(at::kFloat));
-  check_status(tf_flash_decode_f16(Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(),
-                                   ws.data_ptr(), bytes, bh, lkv, d, (int)num_splits, softmax_scale,
-                                   current_stream()),
+  check_status(tf_flash_decode(Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), dtype,
+                               ws.data_ptr(), bytes, bh, lkv, d, (int)num_splits, softmax_scale,
+                               current_stream()),
                "flash_decode");
 }
 
