@@ -145,12 +145,17 @@ TF_API int tf_flash_decode(const void* Q, const void* K, const void* V, void* O,
  * No counterpart in the reference.  It is for callers that cannot allocate device memory: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The device that
  * owns `stream` must be current.  The first call on a device looks up the array's address there
- * (hipGetSymbolAddress); no call allocates or frees.  batch_heads * num_splits above
+ * (hipGetSymbolAddress, which may load the code object): make that first call - or
+ * tf_flash_decode_static_prepare(), which does only the lookup for the current device - OUTSIDE any
+ * stream capture; afterwards a call is two kernel launches and nothing else.  No call allocates or
+ * frees.  The array is part of the library's code object: every process that loads the library
+ * holds it on every GPU it uses, whether or not it calls this entry point.  batch_heads * num_splits above
  * TF_FLASH_DECODE_STATIC_MAX_PARTIALS is rejected with TF_ERR_INVALID_ARG; D must be 128.  Same kernels and
  * bit-identical results as tf_flash_decode_f16.  All calls on one GPU share the one array, so
  * calls that overlap on a GPU (different streams, or threads) race: serialise them. */
 #define TF_FLASH_DECODE_STATIC_MAX_PARTIALS 32768 /* 512 (batch x head) slices x 64 splits */
 TF_API size_t tf_flash_decode_static_max_partials(void);
+TF_API int tf_flash_decode_static_prepare(void);
 TF_API int tf_flash_decode_static_f16(const void* Q, const void* K, const void* V, void* O,
                                       int64_t batch_heads, int64_t Lkv, int64_t D, int num_splits,
                                       double softmax_scale, void* stream);

@@ -77,7 +77,7 @@ def test_decode_argument_validation_and_workspace():
     assert f(p, p, p, p, None, 0, 4, 128, 128, 4, 0.1, None) == _capi.TF_ERR_INVALID_ARG
     assert f(p, p, p, p, p, 16, 4, 128, 128, 4, 0.1, None) == _capi.TF_ERR_INVALID_ARG
     assert b"workspace" in lib.tf_last_error()
-    assert f(p, p, p, p, p, 1 << 20, 4, 128, 64, 4, 0.1, None) == _capi.TF_ERR_UNSUPPORTED
+    assert f(p, p, p, p, p, 1 << 20, 4, 128, 96, 4, 0.1, None) == _capi.TF_ERR_UNSUPPORTED   # 128 and 64 only
     assert f(p, p, p, p, p, 1 << 20, 4, 0, 128, 4, 0.1, None) == _capi.TF_ERR_INVALID_ARG
 
 

@@ -136,6 +136,38 @@ def test_bf16_kernels_exact(m, n, k, p, workspace):
         assert torch.equal(d, c_fused_dtype(a.to(DEV), b.to(DEV), c.to(DEV)).cpu())
 
 
+# Every instance of the plain kernel - n-tiles of 128 / 32, p-tiles of 128 / 64 / 16, k-chunks of
+# 128 / 32, fp16 and bf16 - on problems with several k-chunks (K > KC) and several n-tiles (N > TN)
+# and a ragged row count.  The kernel requests its A fragments from assembly and waits for them by
+# counting requests; a fragment register read before its data has arrived, in any instance, shows as
+# a wrong integer here.  B and C are sparse (+-1 in a few places of every row), so that both products
+# stay small integers, exact even in bf16, while every k-chunk and n-tile contributes to them.
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k", [256, 96])      # k-chunks of 128 (two of them) and of 32 (three)
+@pytest.mark.parametrize("p", [256, 192, 48])  # p-tiles of 128, 64, 16
+@pytest.mark.parametrize("n", [256, 192, 96])  # n-tiles of 128 (two), 32 (six), 32 (three)
+def test_every_plain_kernel_instance_is_exact(dtype, k, p, n):
+    g = torch.Generator().manual_seed(n + p + k)
+    m = 100
+
+    def sparse_rows(rows, cols, per_row):
+        t = torch.zeros(rows, cols)
+        for r in range(rows):
+            idx = torch.randperm(cols, generator=g)[:per_row]
+            t[r, idx] = (torch.randint(0, 2, (per_row,), generator=g) * 2 - 1).float()
+        return t
+    a = torch.randint(-2, 3, (m, k), generator=g).float()
+    b = sparse_rows(n, k, 6)     # every row of B picks six entries of a row of A
+    c = sparse_rows(p, n, 4)     # every row of C picks four entries of the intermediate
+    inter = a @ b.T
+    ref = inter @ c.T
+    assert float(inter.abs().max()) <= 12 and float(ref.abs().max()) <= 48   # integers, exact in bf16 too
+    assert (b.abs().sum(0).reshape(-1, 32).sum(1) > 0).all() and (c.abs().sum(0).reshape(-1, 32).sum(1) > 0).all()
+    for _ in range(2):
+        d = c_fused_dtype(a.to(dtype).to(DEV), b.to(dtype).to(DEV), c.to(dtype).to(DEV)).cpu()
+        assert torch.equal(d.float(), ref)
+
+
 def test_bf16_random_inputs_within_tolerance():
     g = torch.Generator().manual_seed(77)
     a = (torch.randn(512, 128, generator=g) / 11).bfloat16()

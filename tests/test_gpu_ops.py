@@ -161,6 +161,27 @@ def test_flash_attention_ops_for_head_dims_above_128_run_the_header_kernel(d, dv
     assert ok, (r, m)
 
 
+@pytest.mark.parametrize("d,dv,lq,lkv,tq,tkv,causal", [(256, 256, 64, 128, 64, 64, False),
+                                                         (512, 512, 64, 128, 64, 64, False),
+                                                         (384, 384, 128, 256, 128, 128, True),
+                                                         (512, 256, 48, 96, 48, 32, True)])
+def test_flash_attention_ops_shrink_tiles_that_do_not_fit_the_lds(d, dv, lq, lkv, tq, tkv, causal):
+    # Whole-head-dimension tiles of these shapes need more than a CU's 160 KiB of LDS (512 x 512
+    # with 64 x 64 sequence tiles: 192 KiB; 384 x 384 with 128 x 128: 288 KiB).  The launcher cuts
+    # the head dimension into chunks, then the sequence tiles, until they fit.
+    from tilefusion_amd.ops import flash_attention
+    g = torch.Generator().manual_seed(d * 7 + dv)
+    q = torch.randn(2, lq, d, generator=g).half()
+    k = torch.randn(2, lkv, d, generator=g).half()
+    v = torch.randn(2, lkv, dv, generator=g).half()
+    scale = 1.0 / math.sqrt(d)
+    ref = N.attention_ref(q, k, v, scale, causal)
+    o = flash_attention(q.to(DEV), k.transpose(1, 2).contiguous().to(DEV), v.to(DEV), tq, tkv, d, dv, scale, causal)
+    assert o.shape == (2, lq, dv)
+    ok, r, m = N.check_close(o, ref)
+    assert ok, (r, m)
+
+
 def test_flash_attention_key_length_that_cannot_be_padded_is_a_clear_error():
     # above 128 the header kernel is what runs, and its key tiles are 32 wide
     q = torch.randn(16, 160, dtype=torch.float16, device=DEV)

@@ -94,6 +94,25 @@ def test_cache_key_covers_the_contents_of_included_headers(cache_dir, tmp_path_f
     assert len(glob.glob(os.path.join(str(cache_dir), "*.hsaco"))) == 2
 
 
+def test_include_directory_too_deep_to_digest_is_not_cached(cache_dir, tmp_path_factory):
+    # The digest walk is bounded; a header below the bound could change without changing the key,
+    # so nothing compiled against such a directory may be left for a later process to find.
+    from tilefusion_amd.jit import JitCompiler
+    inc = tmp_path_factory.mktemp("deep")
+    deep = inc
+    for level in range(9):
+        deep = deep / f"l{level}"
+    deep.mkdir(parents=True)
+    (deep / "k.hpp").write_text("constexpr float kFactor = 2.0f;\n")
+    rel = "/".join(f"l{level}" for level in range(9))
+    src = f'#include "{rel}/k.hpp"\nextern "C" __global__ void deep_kernel(float* x) {{ x[threadIdx.x] *= kFactor; }}'
+    try:
+        JitCompiler.get_or_compile_kernel("deep_kernel", src, [str(inc)])
+    except RuntimeError as e:
+        assert not torch.cuda.is_available() and "hipModuleLoadData" in str(e)
+    assert not glob.glob(os.path.join(str(cache_dir), "*"))
+
+
 def test_kernel_handles_die_with_clear_cache():
     from tilefusion_amd.jit import JitCompiler, Kernel
     k = Kernel(0, "stale")

@@ -29,6 +29,7 @@ SIGNATURES = {
     "tf_flash_decode_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _i64, _i64, _i64, _i, _d, _vp]),
     "tf_flash_decode": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _sz, _i64, _i64, _i64, _i, _d, _vp]),
     "tf_flash_decode_static_max_partials": (_sz, []),
+    "tf_flash_decode_static_prepare": (_i, []),
     "tf_flash_decode_static_f16": (_i, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i, _d, _vp]),
     "tf_scatter_nd": (_i, [_vp, _vp, _vp, ctypes.POINTER(_i64), _i, _i64, _i, _i, _vp]),
     "tf_jit_compile": (_i, [ctypes.c_char_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_char_p), _i,

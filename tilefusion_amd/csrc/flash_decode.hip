@@ -357,6 +357,11 @@ extern "C" size_t tf_flash_decode_static_max_partials(void) {
   return (size_t)TF_FLASH_DECODE_STATIC_MAX_PARTIALS;
 }
 
+extern "C" int tf_flash_decode_static_prepare(void) {
+  float* unused = nullptr;
+  return tfk::scratch_on_current_device(&unused);
+}
+
 extern "C" int tf_flash_decode_static_f16(const void* Q, const void* K, const void* V, void* O,
                                           int64_t batch_heads, int64_t Lkv, int64_t D,
                                           int num_splits, double softmax_scale, void* stream) {

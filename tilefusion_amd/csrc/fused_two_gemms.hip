@@ -258,12 +258,19 @@ __global__ __launch_bounds__(kThreads) void fused_two_gemms_kernel(
         const char* a_chunk = a_base + (size_t)k0 * 2;
 #pragma unroll
         for (int ks = 0; ks < kKSteps; ++ks)
+          // (early-clobber outputs: a fragment register never doubles as the address register of
+          //  a later request)
           asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3"
-                       : "=v"(af[ks])
+                       : "=&v"(af[ks])
                        : "v"(a_off), "s"(a_chunk), "n"(ks * 64)
                        : "memory");
       }
-      // the A requests are on their way before the arithmetic of the B and C requests starts
+      // the A requests are on their way before the arithmetic of the B and C requests starts.
+      // Between here and the wait below the compiler believes the fragment registers written
+      // although the data is still in flight: nothing in between reads them (only requests and
+      // their scalar address arithmetic are issued), and tests/test_gpu_fused_two_gemms.py::
+      // test_every_plain_kernel_instance_is_exact pins that, for every instance of this kernel and
+      // both element types, on problems with several k-chunks and n-tiles.
       __builtin_amdgcn_sched_barrier(0);
       request_b(n0, k0);
       if (first_chunk) request_c(n0);

@@ -33,9 +33,17 @@ std::string hash_hex(const std::string& s) {
 
 // Digest of every regular file below `dir` (relative name + contents, names sorted): a header
 // edited after a code object was cached must change the cache key.  Bounded in depth and file
-// count so that a stray include path (say "/") cannot stall a compile.
-void collect_files(const std::string& dir, const std::string& rel, int depth, std::vector<std::string>& out) {
-  if (depth > 6 || out.size() > 4096) return;
+// count so that a stray include path (say "/") cannot stall a compile; a walk that hits a bound
+// reports it, and what was compiled against such a directory is not kept on disk.
+constexpr int kMaxWalkDepth = 6;
+constexpr size_t kMaxWalkFiles = 4096;
+
+void collect_files(const std::string& dir, const std::string& rel, int depth, std::vector<std::string>& out,
+                   bool& truncated) {
+  if (depth > kMaxWalkDepth || out.size() >= kMaxWalkFiles) {
+    truncated = true;
+    return;
+  }
   DIR* d = opendir((dir + "/" + rel).c_str());
   if (!d) return;
   std::vector<std::string> names;
@@ -49,14 +57,27 @@ void collect_files(const std::string& dir, const std::string& rel, int depth, st
     const std::string r = rel.empty() ? n : rel + "/" + n;
     struct stat st;
     if (stat((dir + "/" + r).c_str(), &st) != 0) continue;
-    if (S_ISDIR(st.st_mode)) collect_files(dir, r, depth + 1, out);
-    else if (S_ISREG(st.st_mode) && out.size() <= 4096) out.push_back(r);
+    if (S_ISDIR(st.st_mode)) {
+      collect_files(dir, r, depth + 1, out, truncated);
+    } else if (S_ISREG(st.st_mode)) {
+      if (out.size() >= kMaxWalkFiles) {
+        truncated = true;
+        return;
+      }
+      out.push_back(r);
+    }
   }
 }
 
-std::string directory_digest(const std::string& dir) {
+struct DirectoryDigest {
+  std::string hex;
+  bool complete;  // false: some file below the directory is not covered by `hex`
+};
+
+DirectoryDigest directory_digest(const std::string& dir) {
   std::vector<std::string> files;
-  collect_files(dir, "", 0, files);
+  bool truncated = false;
+  collect_files(dir, "", 0, files, truncated);
   std::string material;
   for (const auto& r : files) {
     std::ifstream f(dir + "/" + r, std::ios::binary);
@@ -64,7 +85,35 @@ std::string directory_digest(const std::string& dir) {
     ss << f.rdbuf();
     material += r + "\n" + hash_hex(ss.str()) + "\n";
   }
-  return hash_hex(material);
+  return {hash_hex(material), !truncated};
+}
+
+// Differs between processes (and between runs that re-use a pid): keys that carry it never match
+// a file another process left in the cache directory.
+std::string process_nonce() {
+  static const std::string nonce = [] {
+    struct timespec ts;
+    clock_gettime(CLOCK_REALTIME, &ts);
+    std::ostringstream m;
+    m << (long)getpid() << ':' << (long long)ts.tv_sec << ':' << ts.tv_nsec;
+    return hash_hex(m.str());
+  }();
+  return nonce;
+}
+
+// The fall-back cache directory of a process without a usable home or per-user directory lives
+// as long as the process: its files and the directory itself are removed at exit.
+std::string g_fresh_dir;
+void remove_fresh_dir() {
+  if (g_fresh_dir.empty()) return;
+  if (DIR* d = opendir(g_fresh_dir.c_str())) {
+    while (dirent* e = readdir(d)) {
+      const std::string n = e->d_name;
+      if (n != "." && n != "..") remove((g_fresh_dir + "/" + n).c_str());
+    }
+    closedir(d);
+  }
+  rmdir(g_fresh_dir.c_str());
 }
 
 bool file_exists(const std::string& p) {
@@ -137,6 +186,10 @@ std::string JitCompiler::cache_dir() {
   static const std::string fresh = [] {
     char tmpl[] = "/tmp/tilefusion_mi355x-XXXXXX";
     const char* d = mkdtemp(tmpl);
+    if (d) {
+      g_fresh_dir = d;
+      atexit(remove_fresh_dir);
+    }
     return std::string(d ? d : "");
   }();
   return fresh;
@@ -236,16 +289,22 @@ hipFunction_t JitCompiler::compile_kernel(const std::string& kernel_name, const 
   args.insert(args.end(), compile_args.begin(), compile_args.end());
   std::lock_guard<std::mutex> lock(mutex_);
   // The key covers everything the code object depends on: the source, the arguments, the
-  // CONTENTS of the include directories (digested once per process and directory) and the
-  // compiler and library versions.
+  // CONTENTS of the include directories and the compiler and library versions.  A directory is
+  // digested once per process, the first time a compile names it: a header edited while the
+  // process runs is picked up by the next process, not by this one.  A directory too large to
+  // digest whole makes the result uncacheable: the key then carries a per-process nonce and the
+  // code object is deleted from the cache directory once it is loaded.
   static const std::string toolchain = toolchain_digest();
-  static std::map<std::string, std::string> dir_digests;
+  static std::map<std::string, DirectoryDigest> dir_digests;
   std::string material = hip_source + "\n" + toolchain;
+  bool cacheable = true;
   for (const auto& p : includes) {
     auto it = dir_digests.find(p);
     if (it == dir_digests.end()) it = dir_digests.emplace(p, directory_digest(p)).first;
-    material += "\n-I" + p + "=" + it->second;
+    material += "\n-I" + p + "=" + it->second.hex;
+    cacheable = cacheable && it->second.complete;
   }
+  if (!cacheable) material += "\nnonce=" + process_nonce();
   for (const auto& a : args) material += "\n" + a;
   const std::string key = hash_hex(material);
 
@@ -255,6 +314,7 @@ hipFunction_t JitCompiler::compile_kernel(const std::string& kernel_name, const 
   const std::string object = compile_to_code_object(key, hip_source, includes, args);
   if (object.empty()) return nullptr;
   hipFunction_t fn = load_and_get_kernel(key, object, kernel_name);
+  if (!cacheable) remove(object.c_str());  // the module holds its own copy of the image
   if (fn) kernel_cache_[cache_key] = fn;
   return fn;
 }

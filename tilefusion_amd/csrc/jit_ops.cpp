@@ -68,6 +68,22 @@ int pick_divisor(int64_t n, std::initializer_list<int> candidates) {
   return 0;
 }
 
+// Replaces t by the largest multiple of `unit` below it that divides n and is at least `floor`;
+// false when there is none.
+bool shrink_tile(int& t, int64_t n, int unit, int floor) {
+  for (int c = (t - 1) / unit * unit; c >= floor && c > 0; c -= unit)
+    if (n % c == 0) {
+      t = c;
+      return true;
+    }
+  return false;
+}
+
+// LDS bytes of the header attention kernel: one Q, one K and one V tile of 2-byte elements.
+unsigned attention_lds_bytes(int tq, int tkv, int thqk, int thv) {
+  return (unsigned)(tq * thqk + thqk * tkv + tkv * thv) * 2u;
+}
+
 }  // namespace
 
 bool jit_flash_attention_supports(int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int v_is_transposed) {
@@ -85,6 +101,21 @@ int jit_flash_attention(const void* Q, const void* K, const void* Vt, void* O, i
   if (thv % 16 != 0 || Dv % thv != 0) thv = (int)Dv;
   TFK_REQUIRE(tq > 0 && tkv > 0, TF_ERR_UNSUPPORTED, "flash_attention: no legal tiling for Lq=%lld Lkv=%lld",
               (long long)Lq, (long long)Lkv);
+  // Tiles that do not fit the CU's LDS are shrunk until they do.  The head-dimension chunks go
+  // first (a shorter reduction chunk only re-fetches Q per key tile, a narrower output chunk
+  // repeats Q K^T per chunk), each down to 128 before the sequence tiles go down to 64, then
+  // everything to its smallest legal size.
+  while (attention_lds_bytes(tq, tkv, thqk, thv) > (unsigned)kMaxLdsBytes) {
+    if (thqk > 128 && shrink_tile(thqk, D, 32, 128)) continue;
+    if (thv > 128 && shrink_tile(thv, Dv, 16, 128)) continue;
+    if (tq > 64 && shrink_tile(tq, Lq, 16, 64)) continue;
+    if (tkv > 64 && shrink_tile(tkv, Lkv, 32, 64)) continue;
+    if (shrink_tile(thqk, D, 32, 32)) continue;
+    if (shrink_tile(thv, Dv, 16, 16)) continue;
+    if (shrink_tile(tq, Lq, 16, 16)) continue;
+    if (shrink_tile(tkv, Lkv, 32, 32)) continue;
+    break;  // smallest legal tiles: compile_and_launch reports the LDS need
+  }
   // wavefronts stacked along the query rows: 16 rows each, at most 4
   int wr = tq / 16 > 4 ? 4 : tq / 16;
   while ((tq / wr) % 16 != 0) --wr;
@@ -98,7 +129,7 @@ int jit_flash_attention(const void* Q, const void* K, const void* Vt, void* O, i
       << "extern \"C\" __global__ __launch_bounds__(" << wr * 64 << ") void " << name.str() << "(const " << T
       << "* Q, const " << T << "* K, const " << T << "* V, " << T << "* O) {\n"
       << "  ke_flash_attention<" << T << ", float, " << T << ", Config>(Q, K, V, O);\n}\n";
-  const unsigned lds = (unsigned)(tq * thqk + thqk * tkv + tkv * thv + tq * tkv) * 2u;
+  const unsigned lds = attention_lds_bytes(tq, tkv, thqk, thv);
   void* args[] = {&Q, &K, &Vt, &O};
   return compile_and_launch(name.str(), src.str(), dim3((unsigned)(Lq / tq), (unsigned)(Dv / thv), (unsigned)batch),
                             wr * 64, lds, args, st);
