@@ -1,8 +1,8 @@
-"""Flash-attention forward over head dimensions: the tuned kernels (D = 64, 128; fp16 and bf16)
+"""Flash-attention forward over head dimensions: the tuned kernels (D = 64, 96, 128; fp16 and bf16)
 next to the header macro kernel ke_flash_attention compiled at run time (what any other head
-dimension runs, here D = 96 and D = 32), all through the same entry point
-tf_flash_attention_fwd; and the torch op for those head dimensions, which zero-pads them to the
-next tuned size instead (TFLOP/s count the unpadded problem).  Counterpart of the reference's benchmarks/cpp/flashattention
+dimension runs, here D = 160 and D = 32), all through the same entry point
+tf_flash_attention_fwd; and the torch op, which zero-pads a head dimension below 128 without a
+tuned kernel to the next tuned size instead (TFLOP/s count the unpadded problem).  Counterpart of the reference's benchmarks/cpp/flashattention
 program; every row is checked against an fp32 softmax(QK^T)V of one (batch, head) slice.
 
     python benchmarks/attention/bench.py      # prints a markdown table
@@ -20,10 +20,11 @@ from tilefusion_amd import _capi  # noqa: E402
 BH, S = 32, 4096
 # (head dim, dtype, causal, what runs)
 CASES = [(128, torch.float16, False, "tuned"), (128, torch.float16, True, "tuned"), (128, torch.bfloat16, False, "tuned"),
-         (64, torch.float16, False, "tuned"), (96, torch.float16, False, "header kernel"),
-         (96, torch.float16, True, "header kernel"), (96, torch.bfloat16, False, "header kernel"),
+         (96, torch.float16, False, "tuned"), (96, torch.float16, True, "tuned"), (96, torch.bfloat16, False, "tuned"),
+         (64, torch.float16, False, "tuned"),
+         (160, torch.float16, False, "header kernel"), (160, torch.float16, True, "header kernel"),
          (32, torch.float16, False, "header kernel"),
-         (96, torch.float16, False, "torch op: padded to 128, tuned"), (96, torch.float16, True, "torch op: padded to 128, tuned"),
+         (80, torch.float16, False, "torch op: padded to 96, tuned"), (80, torch.float16, True, "torch op: padded to 96, tuned"),
          (32, torch.float16, False, "torch op: padded to 64, tuned")]
 
 

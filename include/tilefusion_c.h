@@ -95,7 +95,7 @@ TF_API int tf_fused_two_gemms_ws(const void* A, const void* B, const void* C, vo
  * Q [batch, Lq, D]; K [batch, Lkv, D]; V [batch, Lkv, Dv] when v_is_transposed == 0, or
  * [batch, Dv, Lkv] when 1 (what the reference op receives, python/ops/flash_attention.py:74);
  * O [batch, Lq, Dv].  Causal mask: key index > query index is masked
- * (include/cell/mask.hpp:75-82).  (D, Dv) = (128, 128) and (64, 64) run the tuned kernels: any Lq
+ * (include/cell/mask.hpp:75-82).  (D, Dv) = (128, 128), (96, 96) and (64, 64) run the tuned kernels: any Lq
  * and Lkv (a transposed V needs Lkv % 8 == 0 to keep its rows 16-byte aligned).  Other head
  * dimensions are compiled at run time from the header kernel with the caller's tile sizes, as
  * the reference does for every call (src/kernels/flash_attn.cu:16-55): that path needs a
@@ -111,7 +111,7 @@ TF_API int tf_flash_attention_fwd_f16(const void* Q, const void* K, const void* 
                                       int tile_length_kv, int tile_hidden_qk, int tile_hidden_v,
                                       double softmax_scale, int causal, void* stream);
 
-/* The same for fp16 or bf16 (dtype as in tf_gemm).  bf16 with (D, Dv) = (128, 128) or (64, 64) runs
+/* The same for fp16 or bf16 (dtype as in tf_gemm).  bf16 with (D, Dv) = (128, 128), (96, 96) or (64, 64) runs
  * the tuned kernels with the bf16 MFMA, bf16 softmax weights and bf16 output; other head dimensions
  * take the run-time compiled path as above. */
 TF_API int tf_flash_attention_fwd(const void* Q, const void* K, const void* V, void* O, int dtype,

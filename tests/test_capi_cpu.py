@@ -62,7 +62,7 @@ def test_attention_argument_validation():
     p = 0x1000
     f = lib.tf_flash_attention_fwd_f16
     assert f(p, p, None, p, 1, 64, 64, 128, 128, 0, 64, 64, 128, 128, 0.1, 0, None) == _capi.TF_ERR_INVALID_ARG
-    assert f(p, p, p, p, 1, 64, 64, 96, 96, 0, 64, 64, 96, 96, 0.1, 0, None) == _capi.TF_ERR_UNSUPPORTED
+    assert f(p, p, p, p, 1, 64, 64, 80, 80, 0, 64, 64, 80, 80, 0.1, 0, None) == _capi.TF_ERR_UNSUPPORTED
     assert f(p, p, p, p, 1, 64, 64, 128, 128, 0, 48, 64, 128, 128, 0.1, 0, None) == _capi.TF_ERR_INVALID_ARG
     assert f(p, p, p, p, 1, 64, 60, 128, 128, 1, 64, 60, 128, 128, 0.1, 0, None) == _capi.TF_ERR_UNSUPPORTED
     assert f(p, p, p, p, 1, 64, 64, 128, 128, 0, 64, 64, 128, 128, float("nan"), 0, None) == _capi.TF_ERR_INVALID_ARG

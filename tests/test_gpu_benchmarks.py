@@ -77,7 +77,8 @@ def test_attention_head_dim_table_is_correct_on_a_small_problem():
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
     buf = io.StringIO()
-    cases = [(128, torch.float16, True, "tuned"), (64, torch.bfloat16, False, "tuned"),
-             (96, torch.float16, True, "header kernel"), (32, torch.bfloat16, False, "header kernel")]
+    cases = [(128, torch.float16, True, "tuned"), (64, torch.bfloat16, False, "tuned"), (96, torch.float16, True, "tuned"),
+             (160, torch.float16, True, "header kernel"), (32, torch.bfloat16, False, "header kernel"),
+             (80, torch.float16, False, "torch op: padded to 96, tuned")]
     assert mod.run(cases=cases, bh=2, s=512, out=buf), buf.getvalue()
     assert "MISMATCH" not in buf.getvalue()

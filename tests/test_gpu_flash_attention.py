@@ -33,7 +33,8 @@ def test_reference_cases(lq, lkv, causal, v_transposed):
 
 
 @pytest.mark.parametrize("b,lq,lkv,d", [(3, 200, 136, 128), (2, 1, 16, 128), (2, 128, 1000, 128), (1, 513, 513, 128),
-                                        (2, 256, 512, 64), (4, 96, 72, 64), (1, 1024, 2048, 128)])
+                                        (2, 256, 512, 64), (4, 96, 72, 64), (1, 1024, 2048, 128),
+                                        (2, 256, 512, 96), (3, 200, 136, 96), (1, 1024, 1100, 96), (2, 100, 40, 96)])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("v_transposed", [False, True])
 def test_shapes(b, lq, lkv, d, causal, v_transposed):
@@ -63,7 +64,7 @@ def test_short_key_ranges_through_the_eight_wavefront_ring(lkv, causal):
     assert ok, f"rel_l2={r:.3e} max_abs={m:.3e}"
 
 
-@pytest.mark.parametrize("lq,d", [(512, 128), (768, 128), (1024, 64), (300, 128)])
+@pytest.mark.parametrize("lq,d", [(512, 128), (768, 128), (1024, 64), (300, 128), (512, 96), (768, 96)])
 def test_causal_pass_orders(lq, d):
     q, k, v = _inputs(3, lq, lq, d, 77 + lq)
     o = c_attention(q.to(DEV), k.to(DEV), v.to(DEV), True, None, False)
@@ -160,6 +161,7 @@ def test_large_scale_and_large_q_stay_finite():
     (3, 256, 512, 128, False, False), (2, 384, 384, 128, True, False), (2, 200, 333, 128, False, False),
     (2, 100, 100, 128, True, False), (2, 256, 256, 64, True, False), (3, 130, 517, 64, False, False),
     (2, 256, 512, 128, False, True), (2, 320, 320, 64, True, True),
+    (2, 256, 512, 96, False, False), (2, 384, 384, 96, True, False), (2, 130, 520, 96, False, True),
 ])
 def test_bf16_tuned_kernels_match_the_oracle(bh, lq, lkv, d, causal, vt):
     g = torch.Generator().manual_seed(bh * 1000 + lq + lkv + d)
@@ -185,3 +187,24 @@ def test_bf16_and_fp16_kernels_agree_on_inputs_both_can_hold():
     assert N.rel_l2(o16, ref) <= 1e-3
     assert N.rel_l2(ob, ref) <= 4e-3
     assert N.rel_l2(ob.float(), o16.float().cpu()) <= 4e-3
+
+
+def test_head_dimension_96_never_reads_the_padding_of_its_lds_rows():
+    # Head dimension 96 is kept in 128-element LDS rows; the 32 elements of padding hold copies of
+    # the row's last 8 columns (the requests re-fetch the last 16-byte chunk).  Those columns are
+    # made to dominate the scores and the values: a fragment read that strayed into the padding
+    # would count them more than once.
+    g = torch.Generator().manual_seed(96)
+    q = torch.randn(2, 256, 96, generator=g)
+    k = torch.randn(2, 192, 96, generator=g)
+    v = torch.randn(2, 192, 96, generator=g)
+    q[..., 88:] *= 3.0
+    k[..., 88:] *= 3.0
+    v[..., 88:] += 4.0
+    q, k, v = q.half(), k.half(), v.half()
+    for causal in (False, True):
+        for vt in (False, True):
+            vd = v.transpose(1, 2).contiguous() if vt else v
+            o = c_attention(q.to(DEV), k.to(DEV), vd.to(DEV), causal, None, vt)
+            ok, r, m = N.check_close(o, N.attention_ref(q, k, v, causal=causal))
+            assert ok, f"causal={causal} vt={vt}: rel_l2={r:.3e} max_abs={m:.3e}"

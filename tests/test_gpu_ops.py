@@ -126,8 +126,9 @@ def _close_bf16(out, ref):
                                                 (48, 48, 200, 160, True), (32, 16, 64, 96, False)])
 def test_flash_attention_ops_for_head_dims_without_a_tuned_kernel(d, dv, lq, lkv, causal):
     # Head dimensions up to 128 without a tuned kernel are zero-padded by the op to the next tuned
-    # size ((48, 48) -> 64, the others -> 128) and run the tuned kernel, any Lq and Lkv.  Both op
-    # forms (natural and transposed V).
+    # size ((48, 48) and (32, 16) -> 64, (48, 80) -> 96, mixed ones above that -> 128) and run the
+    # tuned kernel, any Lq and Lkv; (96, 96) has a tuned kernel of its own.  Both op forms (natural
+    # and transposed V).
     from tilefusion_amd.ops import flash_attention
     g = torch.Generator().manual_seed(d * 1000 + dv)
     q = torch.randn(2, lq, d, generator=g).half()

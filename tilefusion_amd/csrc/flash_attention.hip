@@ -31,6 +31,10 @@ constexpr int kBN = 64;   // keys per tile
 // LDS ring depth: the 8-wavefront kernel keeps two tiles live (its two wavefront sets are half a
 // tile apart) and three in flight; the 4-wavefront kernel one live and three in flight.
 __host__ __device__ constexpr int ring_stages(int waves) { return waves == 8 ? 5 : 4; }
+// Row pitch (in elements) of a [key][dim] tile in LDS: the next power of two.  The swizzles XOR
+// chunk indices, which needs a power-of-two chunk count, and a 1 KiB request must cover whole
+// rows.  A head dimension of 96 is kept in 128-element rows whose last quarter is never read.
+__host__ __device__ constexpr int lds_pitch(int d) { return d <= 64 ? 64 : 128; }
 
 // K tile [kBN][D] (and a transposed V tile [DV][kBN]): 16 consecutive rows reading one logical
 // 16-byte chunk hit 16 different bank groups.
@@ -113,10 +117,11 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   constexpr int kStages = ring_stages(kWavesT);
   constexpr int kRowsPerWave = 16 * kQB;  // kQB 16-query blocks per wavefront
   constexpr int kBMq = kWavesT * kRowsPerWave;
-  constexpr int kKChunks = D / 8;
-  constexpr int kVChunks = kVT ? kBN / 8 : DV / 8;
-  constexpr int kKBytes = kBN * D * 2;
-  constexpr int kVBytes = kBN * DV * 2;
+  constexpr int DP = lds_pitch(D), DVP = lds_pitch(DV);   // LDS row pitch of the K / natural V tile
+  constexpr int kKChunks = DP / 8;
+  constexpr int kVChunks = kVT ? kBN / 8 : DVP / 8;
+  constexpr int kKBytes = kBN * DP * 2;
+  constexpr int kVBytes = kVT ? DV * kBN * 2 : kBN * DVP * 2;
   constexpr int kStageBytes = kKBytes + kVBytes;
   constexpr int kKB = kBN / 16;   // 16-key blocks per tile (rows of S^T)
   constexpr int kKK = D / 32;     // reduction steps of S^T = K Q^T
@@ -208,7 +213,8 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     const int i = (wave + kWavesT * t) % kKInstr;
     constexpr int kRowsPerInstr = 64 / kKChunks;
     const int row = i * kRowsPerInstr + lane / kKChunks;
-    req_off[t] = (unsigned)(row * D + swz_k<kKChunks>(row, lane % kKChunks) * 8) * 2u;
+    // (a physical chunk whose logical chunk lies beyond D is never read: it re-fetches the last one)
+    req_off[t] = (unsigned)(row * D + min(swz_k<kKChunks>(row, lane % kKChunks), D / 8 - 1) * 8) * 2u;
     req_lds[t] = i * 1024;
   }
 #pragma unroll
@@ -217,7 +223,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
     constexpr int kRowsPerInstr = 64 / kVChunks;
     const int row = i * kRowsPerInstr + lane / kVChunks;
     if constexpr (!kVT)  // V tile: [kBN][DV]
-      req_off[kKPerWave + t] = (unsigned)(row * DV + swz_v<kVChunks>(row, lane % kVChunks) * 8) * 2u;
+      req_off[kKPerWave + t] = (unsigned)(row * DV + min(swz_v<kVChunks>(row, lane % kVChunks), DV / 8 - 1) * 8) * 2u;
     else                 // V^T tile: [DV][kBN] out of a [DV][Lkv] matrix
       req_off[kKPerWave + t] = ((unsigned)row * (unsigned)Lkv + swz_k<kVChunks>(row, lane % kVChunks) * 8) * 2u;
     req_lds[kKPerWave + t] = kKBytes + i * 1024;
@@ -242,7 +248,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       const int i = (wave + kWavesT * r) % kKInstr;
       constexpr int kRowsPerInstr = 64 / kKChunks;
       const int row = i * kRowsPerInstr + lane / kKChunks;
-      const int cc = swz_k<kKChunks>(row, lane % kKChunks);
+      const int cc = min(swz_k<kKChunks>(row, lane % kKChunks), D / 8 - 1);
       const int gr = min(n0 + row, Lkv - 1);
       lds_dma_16B(K + (size_t)gr * D + cc * 8, dst);
     } else {
@@ -250,7 +256,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       constexpr int kRowsPerInstr = 64 / kVChunks;
       const int row = i * kRowsPerInstr + lane / kVChunks;
       if constexpr (!kVT) {
-        const int cc = swz_v<kVChunks>(row, lane % kVChunks);
+        const int cc = min(swz_v<kVChunks>(row, lane % kVChunks), DV / 8 - 1);
         const int gr = min(n0 + row, Lkv - 1);
         lds_dma_16B(V + (size_t)gr * DV + cc * 8, dst);
       } else {
@@ -287,7 +293,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   //   K fragment (kb, kk) - A operand, 16 keys x 32 dims: row 16*kb + lr, logical chunk 4*kk + lg.
   unsigned k_off[kKK];
 #pragma unroll
-  for (int kk = 0; kk < kKK; ++kk) k_off[kk] = lr * D * 2 + swz_k<kKChunks>(lr, 4 * kk + lg) * 16;
+  for (int kk = 0; kk < kKK; ++kk) k_off[kk] = lr * DP * 2 + swz_k<kKChunks>(lr, 4 * kk + lg) * 16;
   //   Reduction step j of the second product covers keys 32*j .. +31; slot t of lane group lg
   //   is key 32*j + 4*lg + t (t < 4) or 32*j + 16 + 4*lg + (t - 4): exactly the keys whose
   //   scores the lane already holds in its accumulators of key blocks 2*j and 2*j + 1.
@@ -304,7 +310,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
 #pragma unroll
     for (int db = 0; db < kDB; ++db) {
       const int col = db * 16 + 4 * (lr & 3);
-      v_off[db] = row_l * DV * 2 + swz_v<kVChunks>(row_l, col / 8) * 16 + (col % 8) * 2;
+      v_off[db] = row_l * DVP * 2 + swz_v<kVChunks>(row_l, col / 8) * 16 + (col % 8) * 2;
     }
   } else {
 #pragma unroll
@@ -345,7 +351,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
   auto k_reads = [&](int buf, int it, int kk) __attribute__((always_inline)) {
     const unsigned ka = opaque(smem_base + (it % kStages) * kStageBytes + k_off[kk]);
 #pragma unroll
-    for (int kb = 0; kb < kKB; ++kb) kf[buf][kb] = lds_read_b128<V8>(ka + kb * 16 * D * 2);
+    for (int kb = 0; kb < kKB; ++kb) kf[buf][kb] = lds_read_b128<V8>(ka + kb * 16 * DP * 2);
   };
   auto v_reads = [&](int buf, int it, int j) __attribute__((always_inline)) {
     const unsigned stage_base = smem_base + (it % kStages) * kStageBytes;
@@ -354,8 +360,8 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       V4 lo, hi;
       if constexpr (!kVT) {
         const unsigned va = opaque(stage_base + v_off[db]) + kKBytes;
-        lo = lds_read_tr4<V4>(va + (32 * j) * DV * 2);
-        hi = lds_read_tr4<V4>(va + (32 * j + 16) * DV * 2);
+        lo = lds_read_tr4<V4>(va + (32 * j) * DVP * 2);
+        hi = lds_read_tr4<V4>(va + (32 * j + 16) * DVP * 2);
       } else {
         lo = lds_read_b64<V4>(opaque(stage_base + v_off[2 * j]) + kKBytes + db * 16 * kBN * 2);
         hi = lds_read_b64<V4>(opaque(stage_base + v_off[2 * j + 1]) + kKBytes + db * 16 * kBN * 2);
@@ -389,7 +395,7 @@ __global__ __launch_bounds__(kWavesT * 64) void flash_attention_fwd_kernel(
       for (int kb = 0; kb < kKB; ++kb) {
 #pragma unroll
         for (int qb = 0; qb < kQB; ++qb) s[kb][qb] = mfma_t<T>(kf[kk & 1][kb], qf[kk][qb], s[kb][qb]);
-        if (kk + 1 < kKK) kf[(kk + 1) & 1][kb] = lds_read_b128<V8>(ka + kb * 16 * D * 2);
+        if (kk + 1 < kKK) kf[(kk + 1) & 1][kb] = lds_read_b128<V8>(ka + kb * 16 * DP * 2);
         if (req_tile >= 0) {
 #pragma unroll
           for (int r = 0; r < kLoadsPerTile; ++r)
@@ -645,7 +651,7 @@ template <typename T, int D, int DV, bool kVT, bool kCausal, int kWavesT, int kQ
 int launch_w(const void* Q, const void* K, const void* V, void* O, int batch, int Lq, int Lkv,
              float scale_log2, hipStream_t st) {
   auto kern = flash_attention_fwd_kernel<T, D, DV, kVT, kCausal, kWavesT, kQB>;
-  constexpr int lds = ring_stages(kWavesT) * (kBN * D * 2 + kBN * DV * 2);
+  constexpr int lds = ring_stages(kWavesT) * (kBN * lds_pitch(D) * 2 + (kVT ? DV * kBN * 2 : kBN * lds_pitch(DV) * 2));
   static_assert(lds <= kMaxLdsBytes, "tiles do not fit in LDS");
   TFK_LDS_OPT_IN(kern, lds);
   constexpr int bm = kWavesT * 16 * kQB;
@@ -708,7 +714,7 @@ int attention_fallback(const char* who, const void* Q, const void* K, const void
                        int64_t batch, int64_t Lq, int64_t Lkv, int64_t D, int64_t Dv, int v_is_transposed,
                        int tq, int tkv, int thqk, int thv, double softmax_scale, int causal, hipStream_t st) {
   TFK_REQUIRE(jit_flash_attention_supports(Lq, Lkv, D, Dv, v_is_transposed), TF_ERR_UNSUPPORTED,
-              "%s: no tuned kernel for head dims (D=%lld, Dv=%lld) (fp16 has 128/128 and 64/64), and the run-time "
+              "%s: no tuned kernel for head dims (D=%lld, Dv=%lld) (128/128, 96/96 and 64/64 have one), and the run-time "
               "compiled kernel needs a transposed V, D %% 32 == 0, Dv %% 16 == 0, Lq %% 16 == 0, Lkv %% 32 == 0 "
               "(got Lq=%lld Lkv=%lld, V %s); the torch op pads and transposes as needed",
               who, (long long)D, (long long)Dv, (long long)Lq, (long long)Lkv,
@@ -729,7 +735,7 @@ extern "C" int tf_flash_attention_fwd_f16(const void* Q, const void* K, const vo
                                     tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale))
     return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const bool tuned = (D == 128 && Dv == 128) || (D == 64 && Dv == 64);
+  const bool tuned = D == Dv && (D == 128 || D == 96 || D == 64);
   if (!tuned)
     return attention_fallback("tf_flash_attention_fwd_f16", Q, K, V, O, TF_DTYPE_F16, batch, Lq, Lkv, D, Dv,
                               v_is_transposed, tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v,
@@ -740,6 +746,9 @@ extern "C" int tf_flash_attention_fwd_f16(const void* Q, const void* K, const vo
   if (D == 128)
     return pick<half_t, 128, 128>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
                                   v_is_transposed != 0, causal != 0, st);
+  if (D == 96)
+    return pick<half_t, 96, 96>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
+                                v_is_transposed != 0, causal != 0, st);
   return pick<half_t, 64, 64>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
                               v_is_transposed != 0, causal != 0, st);
 }
@@ -758,7 +767,7 @@ extern "C" int tf_flash_attention_fwd(const void* Q, const void* K, const void* 
                                     tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale))
     return rc;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const bool tuned = ((D == 128 && Dv == 128) || (D == 64 && Dv == 64)) && (!v_is_transposed || Lkv % 8 == 0);
+  const bool tuned = D == Dv && (D == 128 || D == 96 || D == 64) && (!v_is_transposed || Lkv % 8 == 0);
   if (!tuned)
     return attention_fallback("tf_flash_attention_fwd", Q, K, V, O, dtype, batch, Lq, Lkv, D, Dv, v_is_transposed,
                               tile_length_q, tile_length_kv, tile_hidden_qk, tile_hidden_v, softmax_scale, causal, st);
@@ -767,6 +776,9 @@ extern "C" int tf_flash_attention_fwd(const void* Q, const void* K, const void* 
   if (D == 128)
     return pick<bf16_t, 128, 128>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
                                   v_is_transposed != 0, causal != 0, st);
+  if (D == 96)
+    return pick<bf16_t, 96, 96>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
+                                v_is_transposed != 0, causal != 0, st);
   return pick<bf16_t, 64, 64>(Q, K, V, O, (int)batch, (int)Lq, (int)Lkv, scale_log2,
                               v_is_transposed != 0, causal != 0, st);
 }

@@ -179,13 +179,14 @@ void attention_impl(const at::Tensor& Q, const at::Tensor& K, const at::Tensor& 
   TORCH_CHECK(leading_numel(K, 2) == batch && leading_numel(V, 2) == batch &&
                   leading_numel(O, 2) == batch,
               "batch dimensions must match.");
-  // Head dimensions up to 128 without a tuned kernel are zero-padded to the next tuned size (64 or
-  // 128): zeros change neither the scores nor the kept output columns, and the tuned kernel on
-  // the padded problem is ~1.8x faster than the header kernel compiled at run time on the exact
-  // one (860 against 480 TFLOP/s of useful work at head dimension 96), copies included.
-  const bool tuned = (d == 128 && dv == 128) || (d == 64 && dv == 64);
+  // Head dimensions up to 128 without a tuned kernel are zero-padded to the next tuned size (64,
+  // 96 or 128): zeros change neither the scores nor the kept output columns, and the tuned kernel
+  // on the padded problem is well ahead of the header kernel compiled at run time on the exact
+  // one, copies included.
+  const bool tuned = d == dv && (d == 128 || d == 96 || d == 64);
   if (!tuned && d <= 128 && dv <= 128 && (!v_transposed || lkv % 8 == 0)) {
-    const int64_t hp = (d <= 64 && dv <= 64) ? 64 : 128;
+    const int64_t hmax = std::max(d, dv);
+    const int64_t hp = hmax <= 64 ? 64 : hmax <= 96 ? 96 : 128;
     at::Tensor Qp = at::constant_pad_nd(Q, {0, hp - d}, 0).contiguous();
     at::Tensor Kp = at::constant_pad_nd(K, {0, hp - d}, 0).contiguous();
     at::Tensor Vp = (v_transposed ? at::constant_pad_nd(V, {0, 0, 0, hp - dv}, 0)
