@@ -1,6 +1,7 @@
 """Kernels written against the reference's tile-programming surface drop in: the reference's OWN
-kernel sources - examples/101_gemm/01_gemm_global_reg/gemm.hpp, 02_gemm_all_mem/gemm.hpp and the
-three macro kernels include/kernels/{gemm,fused_two_gemms,flash_attention}_device.cuh - are
+kernel sources - examples/101_gemm/01_gemm_global_reg/gemm.hpp, 02_gemm_all_mem/gemm.hpp, the
+three macro kernels include/kernels/{gemm,fused_two_gemms,flash_attention}_device.cuh and the kernel
+of its copy benchmark, benchmarks/cpp/g2s_copy/tilefusion_copy.cuh - are
 compiled, unmodified and where they lie, against this repository's headers (recipe: oracle/Makefile,
 drivers: tests/cpp/reference_dropin/*.hip) and run on the GPU against the fp32 oracle.
 
@@ -23,7 +24,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REFERENCE = "/root/reference"
 LIB = os.path.join(ROOT, "oracle", "_ref", "libreference_kernels.so")
 SYMBOLS = ["dropin_example_01", "dropin_example_01_shape", "dropin_example_02", "dropin_example_02_shape",
-           "dropin_ke_gemm", "dropin_ke_gemm_shape", "dropin_ke_fused", "dropin_ke_flash"]
+           "dropin_ke_gemm", "dropin_ke_gemm_shape", "dropin_ke_fused", "dropin_ke_flash",
+           "dropin_g2s_copy", "dropin_g2s_copy_shape"]
 DEV = "cuda:0"
 _vp, _i = ctypes.c_void_p, ctypes.c_int
 
@@ -46,12 +48,13 @@ def test_reference_kernel_sources_compile_against_these_headers():
                     reason="the reference tree is not present on this machine")
 def test_only_the_kernel_files_come_from_the_reference():
     # the drivers must see THIS repository's cell/, types/ and util/ headers: list every file the
-    # compiler opens and check that the only ones under the reference are the five kernel sources
+    # compiler opens and check that the only ones under the reference are the six kernel sources
     inc = os.path.join(ROOT, "tilefusion_amd", "include")
     drivers = os.path.join(ROOT, "tests", "cpp", "reference_dropin")
     opened = set()
     for src, ref_inc in [("example_01.hip", "examples/101_gemm/01_gemm_global_reg"),
-                         ("example_02.hip", "examples/101_gemm/02_gemm_all_mem"), ("device_kernels.hip", "include")]:
+                         ("example_02.hip", "examples/101_gemm/02_gemm_all_mem"), ("device_kernels.hip", "include"),
+                         ("g2s_copy.hip", "benchmarks/cpp/g2s_copy")]:
         p = subprocess.run(["/opt/rocm/bin/hipcc", "-std=c++20", "--offload-arch=gfx950", "-fsyntax-only", "-H", "-w",
                             "-I" + inc, "-I" + os.path.join(REFERENCE, ref_inc), "-x", "hip", os.path.join(drivers, src)],
                            capture_output=True, text=True)
@@ -61,7 +64,7 @@ def test_only_the_kernel_files_come_from_the_reference():
                 opened.add(os.path.relpath(line.split()[-1], REFERENCE))
     assert opened == {"examples/101_gemm/01_gemm_global_reg/gemm.hpp", "examples/101_gemm/02_gemm_all_mem/gemm.hpp",
                       "include/kernels/gemm_device.cuh", "include/kernels/fused_two_gemms_device.cuh",
-                      "include/kernels/flash_attention_device.cuh"}
+                      "include/kernels/flash_attention_device.cuh", "benchmarks/cpp/g2s_copy/tilefusion_copy.cuh"}
 
 
 # ---- on the GPU ---------------------------------------------------------------------------------------
@@ -78,6 +81,8 @@ def lib():
         f.argtypes = [_i] + [ctypes.POINTER(_i)] * 3
     lib.dropin_ke_fused.argtypes = [_vp] * 4
     lib.dropin_ke_flash.argtypes = [_i, _vp, _vp, _vp, _vp]
+    lib.dropin_g2s_copy.argtypes = [_i, _vp, _vp]
+    lib.dropin_g2s_copy_shape.argtypes = [_i] + [ctypes.POINTER(_i)] * 2
     return lib
 
 
@@ -157,3 +162,17 @@ def test_reference_ke_flash_attention_runs(lib, variant, lq, causal):
     assert lib.dropin_ke_flash(variant, q.to(DEV).data_ptr(), k.to(DEV).data_ptr(), vt.to(DEV).data_ptr(), o.data_ptr()) == 0
     ref = N.attention_ref(q, k, v, causal=causal)
     assert torch.allclose(o.float().cpu(), ref, atol=1e-2, rtol=1e-2), (N.rel_l2(o, ref), N.max_abs(o, ref))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", range(11))
+def test_reference_g2s_copy_kernel_moves_every_element(lib, variant):
+    # the tiles and wavefront layouts of the reference's sweep (benchmarks/cpp/g2s_copy/main.cu:143-165)
+    # with its source pattern (element i holds i % 2048, :116-117): global -> swizzled shared -> global
+    rows, cols = _i(), _i()
+    lib.dropin_g2s_copy_shape(variant, rows, cols)
+    numel = rows.value * cols.value
+    src = (torch.arange(numel) % 2048).half().to(DEV)
+    dst = torch.full((numel,), float("nan"), dtype=torch.float16, device=DEV)
+    assert lib.dropin_g2s_copy(variant, src.data_ptr(), dst.data_ptr()) == 0
+    assert torch.equal(dst, src)
