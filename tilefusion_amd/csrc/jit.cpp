@@ -7,6 +7,7 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <ctime>
 #include <algorithm>
 #include <fstream>
 #include <map>
